@@ -1,0 +1,88 @@
+"""ctypes binding of libcatccos_mx.so (the C ABI declared in include/catccos_mx.h).
+
+The library is loaded from catccos_amd/lib/; nothing here falls back to another
+implementation: a missing library raises ImportError with the build command.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "lib", "libcatccos_mx.so")
+
+u8p, i32p, f32p, vp = C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p
+u32, i32, u64, sz = C.c_uint32, C.c_int, C.c_uint64, C.c_size_t
+
+
+class FfnWorkspaceLayout(C.Structure):
+    _fields_ = [(n, C.c_size_t) for n in (
+        "src2sorted", "sorted2src", "counts", "routing_scratch", "gmm_meta",
+        "a_codes", "a_scales", "act_codes", "act_scales", "y", "total")]
+
+
+# name -> (restype, argtypes); every symbol include/catccos_mx.h declares
+SIGNATURES = {
+    "cmx_version": (i32, []),
+    "cmx_last_error": (C.c_char_p, []),
+    "cmx_rt_device_count": (i32, [C.POINTER(C.c_int)]),
+    "cmx_rt_set_device": (i32, [i32]),
+    "cmx_rt_malloc": (i32, [C.POINTER(C.c_void_p), sz]),
+    "cmx_rt_free": (i32, [vp]),
+    "cmx_rt_malloc_host": (i32, [C.POINTER(C.c_void_p), sz]),
+    "cmx_rt_free_host": (i32, [vp]),
+    "cmx_rt_memcpy_h2d": (i32, [vp, vp, sz]),
+    "cmx_rt_memcpy_d2h": (i32, [vp, vp, sz]),
+    "cmx_rt_memset": (i32, [vp, i32, sz]),
+    "cmx_rt_stream_create": (i32, [C.POINTER(C.c_void_p)]),
+    "cmx_rt_stream_destroy": (i32, [vp]),
+    "cmx_rt_stream_sync": (i32, [vp]),
+    "cmx_mx_quant": (i32, [vp, u32, u8p, u32, u8p, u32, u32, u32, i32, i32, vp]),
+    "cmx_mx_dequant": (i32, [u8p, u32, u8p, u32, f32p, u32, u32, u32, i32, vp]),
+    "cmx_mx_gemm": (i32, [u8p, u32, u8p, u32, u8p, u32, u8p, u32, vp, u32, u32, u32, u32, i32, i32, vp]),
+    "cmx_mx_gmm_workspace_bytes": (sz, [u32]),
+    "cmx_mx_gmm": (i32, [u8p, u32, u8p, u32, u8p, u8p, vp, u32, i32p, u32, u32, u32, u32, i32, i32, vp, vp]),
+    "cmx_mx_gmm_swiglu_quant": (i32, [u8p, u32, u8p, u32, u8p, u8p, u8p, u32, u8p, u32, vp, i32p, u32, u32, u32, u32,
+                                      vp, vp]),
+    "cmx_moe_routing_workspace_bytes": (sz, [u32, u32]),
+    "cmx_moe_init_routing": (i32, [i32p, u32, u32, u32, i32p, i32p, i32p, vp, vp]),
+    "cmx_packed_row_bytes": (u32, [u32]),
+    "cmx_quant_scatter": (i32, [vp, u32, i32p, u8p, u32, u8p, u32, u32, u32, u32, vp]),
+    "cmx_moe_token_unpermute": (i32, [vp, u32, u32, i32p, f32p, vp, u32, u32, u32, u32, vp]),
+    "catccos_ascend950_symmetric_bytes": (u64, []),
+    "catccos_ascend950_dispatch_ffn_combine_workspace_bytes": (sz, [u32, u32, u32, u32, u32, i32]),
+    "catccos_ascend950_dispatch_ffn_combine": (i32, [u32, vp, u64, u8p, u8p, u8p, u8p, u8p, u8p, u8p, u8p, u8p, u8p,
+                                                     u32, u32, u32, u32, u32, i32]),
+    "cmx_ffn_workspace_layout_get": (i32, [u32, u32, u32, u32, u32, C.POINTER(FfnWorkspaceLayout)]),
+    "cmx_mfma_raw_probe": (i32, [vp, vp, i32p, i32p, f32p, i32, i32, i32, vp]),
+    "cmx_debug_force_tile": (i32, [i32, i32]),
+}
+
+_lib = None
+
+
+def load() -> C.CDLL:
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise ImportError(
+            f"{LIB_PATH} is missing: build it with `python -m catccos_amd.build` (needs hipcc). "
+            "There is no CPU fallback.")
+    lib = C.CDLL(LIB_PATH)
+    for name, (res, args) in SIGNATURES.items():
+        fn = getattr(lib, name)          # AttributeError names the missing symbol
+        fn.restype = res
+        fn.argtypes = args
+    _lib = lib
+    return lib
+
+
+class CmxError(RuntimeError):
+    pass
+
+
+def check(rc: int) -> None:
+    if rc != 0:
+        msg = load().cmx_last_error()
+        raise CmxError(f"libcatccos_mx error {rc}: {msg.decode() if msg else ''}")

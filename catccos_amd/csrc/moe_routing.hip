@@ -1,0 +1,318 @@
+// MoE routing on one device: stable counting sort of (expert, route) pairs, fused MX quantise +
+// scatter of the routed rows, and the weighted top-k combine.  All three are HBM-bound.
+//
+// Sort = histogram per 512-route chunk -> one-workgroup scan (expert-major, chunk-minor, which is
+// exactly the order of a stable sort) -> scatter, where each chunk is owned by one wavefront that
+// ranks equal keys in lane order with ballots, so the result is the unique stable permutation with
+// no global atomics and no dependence on scheduling.
+#include "mx_common.h"
+
+namespace cmx {
+namespace {
+
+constexpr uint32_t kChunk = 512;   // routes per wavefront-owned chunk
+
+__global__ __launch_bounds__(64) void route_hist_kernel(const int32_t* __restrict__ keys, uint32_t routes,
+                                                         uint32_t experts, uint32_t* __restrict__ hist) {
+    extern __shared__ uint32_t sh[];
+    for (uint32_t e = threadIdx.x; e < experts; e += 64) sh[e] = 0;
+    __syncthreads();
+    const uint32_t base = blockIdx.x * kChunk;
+    for (uint32_t i = threadIdx.x; i < kChunk; i += 64) {
+        const uint32_t r = base + i;
+        if (r < routes) {
+            const int32_t k = keys[r];
+            if (k >= 0 && (uint32_t)k < experts) atomicAdd(&sh[k], 1u);
+        }
+    }
+    __syncthreads();
+    for (uint32_t e = threadIdx.x; e < experts; e += 64) hist[(size_t)blockIdx.x * experts + e] = sh[e];
+}
+
+// hist[c][e] -> offset[c][e] = (rows of experts < e) + (rows of expert e in chunks < c); counts[e].
+__global__ __launch_bounds__(1024) void route_scan_kernel(uint32_t* __restrict__ hist, uint32_t chunks, uint32_t experts,
+                                                           int32_t* __restrict__ counts) {
+    extern __shared__ uint32_t sh[];            // [experts] totals, then [1024] partials
+    uint32_t* tot = sh;
+    uint32_t* part = sh + experts;
+    for (uint32_t e = threadIdx.x; e < experts; e += blockDim.x) {
+        uint32_t run = 0;
+        for (uint32_t c = 0; c < chunks; ++c) {
+            const uint32_t h = hist[(size_t)c * experts + e];
+            hist[(size_t)c * experts + e] = run;
+            run += h;
+        }
+        tot[e] = run;
+        counts[e] = (int32_t)run;
+    }
+    __syncthreads();
+    // exclusive scan of tot[] over experts: contiguous segment per thread + scan of the partials
+    const uint32_t seg = (experts + blockDim.x - 1) / blockDim.x;
+    const uint32_t lo = threadIdx.x * seg;
+    uint32_t s = 0;
+    for (uint32_t e = lo; e < lo + seg && e < experts; ++e) s += tot[e];
+    part[threadIdx.x] = s;
+    __syncthreads();
+    for (uint32_t d = 1; d < blockDim.x; d <<= 1) {
+        uint32_t v = threadIdx.x >= d ? part[threadIdx.x - d] : 0;
+        __syncthreads();
+        part[threadIdx.x] += v;
+        __syncthreads();
+    }
+    uint32_t run = threadIdx.x ? part[threadIdx.x - 1] : 0;
+    for (uint32_t e = lo; e < lo + seg && e < experts; ++e) {
+        const uint32_t t = tot[e];
+        tot[e] = run;
+        run += t;
+    }
+    __syncthreads();
+    for (uint32_t e = threadIdx.x; e < experts; e += blockDim.x) {
+        const uint32_t b = tot[e];
+        for (uint32_t c = 0; c < chunks; ++c) hist[(size_t)c * experts + e] += b;
+    }
+}
+
+__global__ __launch_bounds__(64) void route_scatter_kernel(const int32_t* __restrict__ keys, uint32_t routes,
+                                                            uint32_t experts, uint32_t key_bits,
+                                                            const uint32_t* __restrict__ offset,
+                                                            int32_t* __restrict__ sorted2src,
+                                                            int32_t* __restrict__ src2sorted) {
+    extern __shared__ uint32_t off[];
+    const uint32_t lane = threadIdx.x;
+    for (uint32_t e = lane; e < experts; e += 64) off[e] = offset[(size_t)blockIdx.x * experts + e];
+    __syncthreads();
+    const uint32_t base = blockIdx.x * kChunk;
+    for (uint32_t i = 0; i < kChunk; i += 64) {
+        const uint32_t r = base + i + lane;
+        int32_t k = -1;
+        if (r < routes) {
+            k = keys[r];
+            if (k < 0 || (uint32_t)k >= experts) k = -1;
+        }
+        const bool live = k >= 0;
+        unsigned long long same = __ballot(live);
+        for (uint32_t b = 0; b < key_bits; ++b) {
+            const unsigned long long m = __ballot(live && ((k >> b) & 1));
+            same &= ((k >> b) & 1) ? m : ~m;
+        }
+        if (live) {
+            const uint32_t rank = __popcll(same & ((1ull << lane) - 1ull));
+            const uint32_t pos = off[k] + rank;
+            sorted2src[pos] = (int32_t)r;
+            src2sorted[r] = (int32_t)pos;
+        } else if (r < routes) {
+            src2sorted[r] = -1;
+        }
+        __syncthreads();
+        if (live && lane == 63u - (uint32_t)__clzll(same)) off[k] += (uint32_t)__popcll(same);
+        __syncthreads();
+    }
+}
+
+// ---- fused quantise + scatter -------------------------------------------------------------------
+__device__ __forceinline__ uint32_t quad_max(uint32_t v) {
+    uint32_t t = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0xB1, 0xF, 0xF, true);
+    v = v > t ? v : t;
+    t = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x4E, 0xF, 0xF, true);
+    return v > t ? v : t;
+}
+
+// Four lanes per MX block as in the plain quantizer; k % 32 == 0, rows 16-byte aligned.
+__global__ __launch_bounds__(256) void quant_scatter_kernel(const uint16_t* __restrict__ x, uint32_t ld_x,
+                                                             const int32_t* __restrict__ src2sorted,
+                                                             uint8_t* __restrict__ out_codes, uint32_t ld_out,
+                                                             uint8_t* __restrict__ out_scales, uint32_t ld_outs,
+                                                             uint32_t tokens, uint32_t k, uint32_t top_k, uint32_t nb,
+                                                             uint32_t total_blocks) {
+    const uint32_t q = threadIdx.x & 3u;
+    const uint32_t b = blockIdx.x * 64 + (threadIdx.x >> 2);
+    const bool live = b < total_blocks;
+    const uint32_t row = live ? b / nb : 0;
+    const uint32_t kb = live ? b - row * nb : 0;
+    const uint32_t col = kb * 32 + q * 8;
+    uint4 raw = make_uint4(0, 0, 0, 0);
+    if (live) raw = *reinterpret_cast<const uint4*>(x + (size_t)row * ld_x + col);
+    uint32_t d[4] = {raw.x, raw.y, raw.z, raw.w};
+    uint32_t amax = 0;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const uint32_t a = d[i] & 0x7FFF7FFFu;
+        const uint32_t lo = a & 0xFFFFu, hi = a >> 16;
+        amax = amax > lo ? amax : lo;
+        amax = amax > hi ? amax : hi;
+    }
+    amax = quad_max(amax);
+    const int e = block_exp_from_bf16_amax(amax, kEmaxE4M3);
+    float y[8];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        y[2 * i] = clamp_abs(ldexpf(__uint_as_float(d[i] << 16), -e), 448.0f);
+        y[2 * i + 1] = clamp_abs(ldexpf(__uint_as_float(d[i] & 0xFFFF0000u), -e), 448.0f);
+    }
+    if (!live) return;
+    uint32_t w0 = cvt_pk_e4m3(y[0], y[1], 0u, false);
+    w0 = cvt_pk_e4m3(y[2], y[3], w0, true);
+    uint32_t w1 = cvt_pk_e4m3(y[4], y[5], 0u, false);
+    w1 = cvt_pk_e4m3(y[6], y[7], w1, true);
+    const uint8_t sbyte = (uint8_t)(e + 127);
+    const bool pad = (kb == nb - 1) && (nb & 1u);
+    for (uint32_t r = 0; r < top_k; ++r) {
+        const int32_t dst = src2sorted[(size_t)row * top_k + r];
+        if (dst < 0) continue;
+        *reinterpret_cast<uint2*>(out_codes + (size_t)dst * ld_out + col) = make_uint2(w0, w1);
+        if (q == 0) {
+            uint8_t* s = out_scales + (size_t)dst * ld_outs;
+            s[kb] = sbyte;
+            if (pad) s[nb] = 127;
+        }
+    }
+}
+
+// ---- weighted top-k combine -----------------------------------------------------------------------
+// One workgroup per token; a lane owns 8 consecutive hidden elements per step.
+template <int KMAX>
+__global__ __launch_bounds__(256) void unpermute_kernel(const uint16_t* __restrict__ y, uint32_t ld_y, uint32_t rows,
+                                                         const int32_t* __restrict__ src2sorted,
+                                                         const float* __restrict__ probs, uint16_t* __restrict__ out,
+                                                         uint32_t ld_out, uint32_t hidden, uint32_t top_k) {
+    const uint32_t t = blockIdx.x;
+    __shared__ int32_t s_idx[KMAX];
+    __shared__ float s_w[KMAX];
+    if (threadIdx.x < top_k) {
+        s_idx[threadIdx.x] = src2sorted[(size_t)t * top_k + threadIdx.x];
+        s_w[threadIdx.x] = probs[(size_t)t * top_k + threadIdx.x];
+    }
+    __syncthreads();
+    const uint32_t nvec = hidden >> 3;
+    for (uint32_t v = threadIdx.x; v < nvec; v += blockDim.x) {
+        float acc[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) acc[i] = 0.0f;
+        for (uint32_t k0 = 0; k0 < top_k; k0 += 8) {
+            uint4 raw[8];
+            bool ok[8];
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                const uint32_t k = k0 + j;
+                const int32_t r = k < top_k ? s_idx[k] : -1;
+                ok[j] = r >= 0 && (uint32_t)r < rows;
+                raw[j] = ok[j] ? *reinterpret_cast<const uint4*>(y + (size_t)r * ld_y + v * 8) : make_uint4(0, 0, 0, 0);
+            }
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                const uint32_t k = k0 + j;
+                if (k >= top_k) break;
+                const float w = s_w[k];
+                const uint32_t dd[4] = {raw[j].x, raw[j].y, raw[j].z, raw[j].w};
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    // separate multiply and add (no fused multiply-add): matches Muls then Add in fp32
+                    float t0 = ok[j] ? __fmul_rn(__uint_as_float(dd[i] << 16), w) : 0.0f;
+                    float t1 = ok[j] ? __fmul_rn(__uint_as_float(dd[i] & 0xFFFF0000u), w) : 0.0f;
+                    acc[2 * i] = k == 0 ? t0 : __fadd_rn(acc[2 * i], t0);
+                    acc[2 * i + 1] = k == 0 ? t1 : __fadd_rn(acc[2 * i + 1], t1);
+                }
+            }
+        }
+        uint32_t o[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) o[i] = f32_to_bf16(acc[2 * i]) | (f32_to_bf16(acc[2 * i + 1]) << 16);
+        *reinterpret_cast<uint4*>(out + (size_t)t * ld_out + v * 8) = make_uint4(o[0], o[1], o[2], o[3]);
+    }
+    // ragged tail (hidden % 8 != 0)
+    for (uint32_t c = (nvec << 3) + threadIdx.x; c < hidden; c += blockDim.x) {
+        float acc = 0.0f;
+        for (uint32_t k = 0; k < top_k; ++k) {
+            const int32_t r = s_idx[k];
+            const bool ok = r >= 0 && (uint32_t)r < rows;
+            const float term = ok ? __fmul_rn(bf16_to_f32(y[(size_t)r * ld_y + c]), s_w[k]) : 0.0f;
+            acc = k == 0 ? term : __fadd_rn(acc, term);
+        }
+        out[(size_t)t * ld_out + c] = (uint16_t)f32_to_bf16(acc);
+    }
+}
+
+constexpr int kMaxTopK = 64;
+
+__global__ void fill_i32_kernel(int32_t* p, uint32_t n, int32_t v) {
+    const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) p[i] = v;
+}
+
+}  // namespace
+}  // namespace cmx
+
+extern "C" size_t cmx_moe_routing_workspace_bytes(uint32_t routes, uint32_t experts) {
+    const size_t chunks = (routes + cmx::kChunk - 1) / cmx::kChunk;
+    return cmx::round_up_sz((chunks ? chunks : 1) * (size_t)experts * sizeof(uint32_t), 256);
+}
+
+extern "C" int cmx_moe_init_routing(const int32_t* expert_idx, uint32_t tokens, uint32_t top_k, uint32_t experts,
+                                    int32_t* sorted2src, int32_t* src2sorted, int32_t* counts, void* workspace,
+                                    cmx_stream_t stream) {
+    using namespace cmx;
+    CMX_REQUIRE(expert_idx && sorted2src && src2sorted && counts && workspace, "null pointer");
+    CMX_REQUIRE(experts > 0 && experts <= 8192, "experts must be in [1, 8192]");
+    CMX_REQUIRE(top_k > 0, "top_k must be positive");
+    CMX_REQUIRE((uint64_t)tokens * top_k < (1ull << 31), "too many routes");
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const uint32_t routes = tokens * top_k;
+    const uint32_t chunks = ceil_div(routes, kChunk);
+    uint32_t* hist = static_cast<uint32_t*>(workspace);
+    if (routes == 0) {
+        hipLaunchKernelGGL(fill_i32_kernel, dim3(ceil_div(experts, 256)), dim3(256), 0, s, counts, experts, 0);
+        CMX_LAUNCH_CHECK();
+        return CMX_OK;
+    }
+    uint32_t key_bits = 0;
+    while ((1u << key_bits) < experts) ++key_bits;
+    hipLaunchKernelGGL(route_hist_kernel, dim3(chunks), dim3(64), experts * sizeof(uint32_t), s, expert_idx, routes,
+                       experts, hist);
+    CMX_LAUNCH_CHECK();
+    hipLaunchKernelGGL(route_scan_kernel, dim3(1), dim3(1024), (experts + 1024) * sizeof(uint32_t), s, hist, chunks,
+                       experts, counts);
+    CMX_LAUNCH_CHECK();
+    hipLaunchKernelGGL(route_scatter_kernel, dim3(chunks), dim3(64), experts * sizeof(uint32_t), s, expert_idx, routes,
+                       experts, key_bits, hist, sorted2src, src2sorted);
+    CMX_LAUNCH_CHECK();
+    return CMX_OK;
+}
+
+extern "C" uint32_t cmx_packed_row_bytes(uint32_t k) { return cmx::round_up(k + cmx::scale_cols(k), 32); }
+
+extern "C" int cmx_quant_scatter(const void* x, uint32_t ld_x, const int32_t* src2sorted, uint8_t* out_codes,
+                                 uint32_t ld_out, uint8_t* out_scales, uint32_t ld_outs, uint32_t tokens, uint32_t k,
+                                 uint32_t top_k, cmx_stream_t stream) {
+    using namespace cmx;
+    CMX_REQUIRE(x && src2sorted && out_codes && out_scales, "null pointer");
+    if (tokens == 0 || k == 0 || top_k == 0) return CMX_OK;
+    CMX_REQUIRE(k % 32 == 0, "k must be a multiple of 32");
+    CMX_REQUIRE(ld_x >= k && ld_x % 8 == 0 && aligned16(x), "input rows must be 16-byte aligned");
+    CMX_REQUIRE(ld_out >= k && ld_out % 8 == 0 && (reinterpret_cast<uintptr_t>(out_codes) & 7u) == 0,
+                "output rows must be 8-byte aligned");
+    CMX_REQUIRE(ld_outs >= scale_cols(k), "scale pitch too small");
+    const uint32_t nb = k / 32;
+    CMX_REQUIRE((uint64_t)tokens * nb < (1ull << 32), "too many blocks for one launch");
+    const uint32_t total = tokens * nb;
+    hipLaunchKernelGGL(quant_scatter_kernel, dim3(ceil_div(total, 64)), dim3(256), 0, static_cast<hipStream_t>(stream),
+                       static_cast<const uint16_t*>(x), ld_x, src2sorted, out_codes, ld_out, out_scales, ld_outs, tokens,
+                       k, top_k, nb, total);
+    CMX_LAUNCH_CHECK();
+    return CMX_OK;
+}
+
+extern "C" int cmx_moe_token_unpermute(const void* y, uint32_t ld_y, uint32_t rows, const int32_t* src2sorted,
+                                       const float* probs, void* out, uint32_t ld_out, uint32_t tokens,
+                                       uint32_t hidden, uint32_t top_k, cmx_stream_t stream) {
+    using namespace cmx;
+    CMX_REQUIRE(y && src2sorted && probs && out, "null pointer");
+    if (tokens == 0 || hidden == 0) return CMX_OK;
+    CMX_REQUIRE(top_k > 0 && top_k <= (uint32_t)kMaxTopK, "top_k must be in [1, 64]");
+    CMX_REQUIRE(ld_y >= hidden && ld_out >= hidden, "row pitch smaller than a row");
+    CMX_REQUIRE(ld_y % 8 == 0 && ld_out % 8 == 0 && aligned16(y) && aligned16(out), "rows must be 16-byte aligned");
+    hipLaunchKernelGGL((unpermute_kernel<kMaxTopK>), dim3(tokens), dim3(256), 0, static_cast<hipStream_t>(stream),
+                       static_cast<const uint16_t*>(y), ld_y, rows, src2sorted, probs, static_cast<uint16_t*>(out),
+                       ld_out, hidden, top_k);
+    CMX_LAUNCH_CHECK();
+    return CMX_OK;
+}

@@ -1,0 +1,614 @@
+// Block-scaled MX matmul for gfx950 on v_mfma_scale_f32_32x32x64_f8f6f4.
+//
+//   C[m, n] = sum_k deq(A)[m, k] * deq(W)[n, k]        A = activations, W = transposed weights
+//
+// Both operands are K-contiguous, which is what the scaled MFMA wants: per step a lane feeds two
+// 16-byte runs of one row (FP4: one run = a whole 32-block) plus that row's E8M0 byte for the
+// 32-block its half-wave owns.  The weights
+// are the MFMA's first operand and the activations the second, so an accumulator register quad
+// holds four consecutive n for one m: stores are 8-byte vectors and the SwiGLU/requant epilogue
+// finds a whole 32-wide MX block of one activation row in two lanes (l and l^32).
+//
+// One workgroup (256 threads = 4 wavefronts) owns a TW x TM tile (weight rows x activation rows)
+// and walks K in 128-byte slabs through a two-stage LDS ring: while the MFMAs consume slab i
+// the global loads of slab i+1 are in flight in registers.  A/W tiles are stored with a 16-byte
+// chunk XOR swizzle so both the 16-byte row-strided MFMA operand reads and the staging writes are
+// bank-conflict free; the per-row scale dwords of the slab ride along in LDS.
+//
+// Ragged expert groups: a tiny prologue kernel turns the device-resident group sizes into row
+// offsets and a prefix of m-tiles; each workgroup binary-searches its (group, n-tile, m-tile) from
+// that prefix, so no host synchronisation is needed and empty groups cost nothing.  Workgroup ids
+// are remapped so that each XCD (ids congruent mod 8) walks a contiguous run of tiles that share
+// weight panels in its own L2.
+#include "mx_common.h"
+
+namespace cmx {
+
+namespace {
+
+constexpr int kThreads = 256;
+constexpr int kSlabBytes = 128;     // K bytes per LDS slab and row
+constexpr int kChunks = kSlabBytes / 16;
+constexpr int kXcds = 8;
+
+enum Epilogue { kEpiStore = 0, kEpiSwigluQuant = 1 };
+
+struct GemmParams {
+    const uint8_t* a;        // activations codes
+    const uint8_t* a_scale;
+    const uint8_t* w;        // weights codes [groups][n][ldw]
+    const uint8_t* w_scale;  // [groups][n][ld_ws]
+    void* c;
+    uint8_t* act_codes;
+    uint8_t* act_scales;
+    uint16_t* act_bf16;
+    const int32_t* row_off;     // [groups+1] (grouped) or null (dense)
+    const int32_t* tile_pref;   // [groups+1] prefix of m-tiles (grouped) or null
+    uint32_t lda, ld_as, ldw, ld_ws, ldc, ld_act, ld_acts;
+    uint32_t m, n, kbytes, kblocks;   // kblocks = K/32
+    uint32_t groups, w_tiles;
+    int out_type;
+    int scale_vec;   // scale rows are 4-byte aligned: one dword load per row and slab
+};
+
+__device__ __forceinline__ uint32_t swz(uint32_t row, uint32_t chunk) {
+    return chunk ^ ((row & 7u) ^ ((row >> 3) & 1u));
+}
+
+__device__ __forceinline__ v4f to_v4(const v16f& v, int q) {
+    v4f r = {v[4 * q], v[4 * q + 1], v[4 * q + 2], v[4 * q + 3]};
+    return r;
+}
+
+template <int FMT>
+__device__ __forceinline__ v16f mfma(v8i w, v8i a, v16f c, int opsel_tag, int sw, int sa);
+
+// opsel picks which byte of the lane's scale register feeds the MFMA (same byte for both operands here)
+#define CMX_MFMA_CASE(fmtcode, sel) \
+    __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(w, a, c, fmtcode, fmtcode, sel, sw, sel, sa)
+
+template <>
+__device__ __forceinline__ v16f mfma<CMX_FMT_E4M3>(v8i w, v8i a, v16f c, int sel, int sw, int sa) {
+    switch (sel) {
+        case 0: return CMX_MFMA_CASE(0, 0);
+        case 1: return CMX_MFMA_CASE(0, 1);
+        case 2: return CMX_MFMA_CASE(0, 2);
+        default: return CMX_MFMA_CASE(0, 3);
+    }
+}
+template <>
+__device__ __forceinline__ v16f mfma<CMX_FMT_E5M2>(v8i w, v8i a, v16f c, int sel, int sw, int sa) {
+    switch (sel) {
+        case 0: return CMX_MFMA_CASE(1, 0);
+        case 1: return CMX_MFMA_CASE(1, 1);
+        case 2: return CMX_MFMA_CASE(1, 2);
+        default: return CMX_MFMA_CASE(1, 3);
+    }
+}
+template <>
+__device__ __forceinline__ v16f mfma<CMX_FMT_E2M1>(v8i w, v8i a, v16f c, int sel, int sw, int sa) {
+    switch (sel) {
+        case 0: return CMX_MFMA_CASE(4, 0);
+        case 1: return CMX_MFMA_CASE(4, 1);
+        case 2: return CMX_MFMA_CASE(4, 2);
+        default: return CMX_MFMA_CASE(4, 3);
+    }
+}
+
+__device__ __forceinline__ float silu_mul(float g, float u) {
+    float s = 1.0f / (1.0f + __expf(-g));
+    return (g * s) * u;
+}
+
+// TW/TM: tile rows (weights / activations); WW x WM wavefront grid over the tile.
+template <int FMT, int TW, int TM, int WW, int WM, int EPI>
+__global__ __launch_bounds__(kThreads) void mx_gemm_kernel(const GemmParams p) {
+    static_assert(WW * WM == 4, "four wavefronts per workgroup");
+    constexpr bool kFp4 = FMT == CMX_FMT_E2M1;
+    constexpr int kSub = kFp4 ? 4 : 2;                 // MFMA steps (64 K elements each) per slab
+    constexpr int kScaleDw = kFp4 ? 2 : 1;             // scale dwords per row per slab
+    constexpr int FW = TW / WW / 32;                   // 32-row fragments per wavefront, weights
+    constexpr int FM = TM / WM / 32;                   // activations
+    constexpr int kWLoads = TW / 32;                   // 16-byte chunks per thread per slab
+    constexpr int kALoads = TM / 32;
+    static_assert(EPI == kEpiStore || (FW % 2 == 0), "gate/up fragments come in pairs");
+    constexpr int kStageBytes = (TW + TM) * kSlabBytes + (TW + TM) * 4 * kScaleDw;
+
+    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+
+    const uint32_t tid = threadIdx.x;
+    const uint32_t lane = tid & 63u;
+    const uint32_t wave = tid >> 6;
+    const uint32_t ww = wave % WW, wm = wave / WW;
+
+    // ---- which tile -------------------------------------------------------------------------
+    uint32_t total_tiles, g = 0, mt, wt, row0, rows_valid;
+    {
+        const uint32_t grouped = p.row_off != nullptr;
+        uint32_t m_tiles_all = grouped ? (uint32_t)p.tile_pref[p.groups] : (p.m + TM - 1) / TM;
+        total_tiles = m_tiles_all * p.w_tiles;
+        const uint32_t bid = blockIdx.x;
+        if (bid >= total_tiles) return;
+        // XCD-aware remap: ids congruent mod 8 run on one XCD; give each a contiguous run.
+        const uint32_t x = bid % kXcds, j = bid / kXcds;
+        const uint32_t base = total_tiles / kXcds, rem = total_tiles % kXcds;
+        const uint32_t L = x * base + (x < rem ? x : rem) + j;
+        if (grouped) {
+            // find g with tile_pref[g]*w_tiles <= L < tile_pref[g+1]*w_tiles
+            uint32_t lo = 0, hi = p.groups;
+            while (hi - lo > 1) {
+                uint32_t mid = (lo + hi) >> 1;
+                if ((uint32_t)p.tile_pref[mid] * p.w_tiles <= L) lo = mid; else hi = mid;
+            }
+            g = lo;
+            const uint32_t tp = (uint32_t)p.tile_pref[g];
+            const uint32_t mtg = (uint32_t)p.tile_pref[g + 1] - tp;
+            const uint32_t local = L - tp * p.w_tiles;
+            mt = local % mtg;
+            wt = local / mtg;
+            const uint32_t r_begin = (uint32_t)p.row_off[g], r_end = (uint32_t)p.row_off[g + 1];
+            row0 = r_begin + mt * TM;
+            rows_valid = r_end - row0 < (uint32_t)TM ? r_end - row0 : (uint32_t)TM;
+        } else {
+            // groups of 4 m-tiles share a run of weight tiles
+            const uint32_t m_tiles = m_tiles_all;
+            const uint32_t band = 4;
+            const uint32_t per_band = band * p.w_tiles;
+            const uint32_t b = L / per_band, within = L % per_band;
+            const uint32_t band_rows = (m_tiles - b * band) < band ? (m_tiles - b * band) : band;
+            mt = b * band + within % band_rows;
+            wt = within / band_rows;
+            row0 = mt * TM;
+            rows_valid = p.m - row0 < (uint32_t)TM ? p.m - row0 : (uint32_t)TM;
+        }
+    }
+
+    // ---- global -> LDS staging assignments -----------------------------------------------------
+    const uint32_t ld_chunk = tid & 7u;        // 16-byte chunk inside the slab
+    const uint32_t ld_row = tid >> 3;          // + 32*j
+    const uint8_t* wg = p.w + (size_t)g * p.n * p.ldw;
+    const uint8_t* wsg = p.w_scale + (size_t)g * p.n * p.ld_ws;
+
+    // global weight row of LDS tile row r
+    auto wrow_of = [&](uint32_t r) -> uint32_t {
+        uint32_t gr;
+        if (EPI == kEpiSwigluQuant) {
+            const uint32_t half = p.n >> 1;
+            uint32_t rr = r < TW / 2 ? wt * (TW / 2) + r : wt * (TW / 2) + (r - TW / 2);
+            rr = rr < half ? rr : half - 1;
+            gr = r < TW / 2 ? rr : half + rr;
+        } else {
+            gr = wt * TW + r;
+            gr = gr < p.n ? gr : p.n - 1;
+        }
+        return gr;
+    };
+    auto arow_of = [&](uint32_t r) -> uint32_t { return row0 + (r < rows_valid ? r : rows_valid - 1); };
+
+    const uint8_t* wptr[kWLoads];
+    const uint8_t* aptr[kALoads];
+#pragma unroll
+    for (int j = 0; j < kWLoads; ++j) wptr[j] = wg + (size_t)wrow_of(ld_row + 32 * j) * p.ldw + ld_chunk * 16;
+#pragma unroll
+    for (int j = 0; j < kALoads; ++j) aptr[j] = p.a + (size_t)arow_of(ld_row + 32 * j) * p.lda + ld_chunk * 16;
+    // scale rows: thread t serves weight row t (t < TW) and activation row t (t < TM)
+    const uint8_t* wsptr = wsg + (size_t)wrow_of(tid < TW ? tid : 0) * p.ld_ws;
+    const uint8_t* asptr = p.a_scale + (size_t)arow_of(tid < TM ? tid : 0) * p.ld_as;
+
+    const uint32_t nslab = (p.kbytes + kSlabBytes - 1) / kSlabBytes;
+    const uint32_t blocks_per_slab = 4 * kScaleDw;
+
+    uint4 wreg[kWLoads], areg[kALoads];
+    uint32_t wsreg[kScaleDw], asreg[kScaleDw];
+
+    auto load_scale_dw = [&](const uint8_t* rowp, uint32_t blk0) -> uint32_t {
+        // four consecutive scale bytes starting at block blk0; beyond K the scale is 1.0
+        if (p.scale_vec && blk0 + 4 <= p.kblocks) return *reinterpret_cast<const uint32_t*>(rowp + blk0);
+        uint32_t v = 0x7F7F7F7Fu;
+        for (uint32_t i = 0; i < 4; ++i)
+            if (blk0 + i < p.kblocks) v = (v & ~(0xFFu << (8 * i))) | ((uint32_t)rowp[blk0 + i] << (8 * i));
+        return v;
+    };
+    auto load_global = [&](uint32_t slab) {
+        const uint32_t kb = slab * kSlabBytes + ld_chunk * 16;
+        const bool in = kb < p.kbytes;
+#pragma unroll
+        for (int j = 0; j < kWLoads; ++j)
+            wreg[j] = in ? *reinterpret_cast<const uint4*>(wptr[j] + (size_t)slab * kSlabBytes) : make_uint4(0, 0, 0, 0);
+#pragma unroll
+        for (int j = 0; j < kALoads; ++j)
+            areg[j] = in ? *reinterpret_cast<const uint4*>(aptr[j] + (size_t)slab * kSlabBytes) : make_uint4(0, 0, 0, 0);
+#pragma unroll
+        for (int d = 0; d < kScaleDw; ++d) {
+            const uint32_t blk0 = slab * blocks_per_slab + 4 * d;
+            if (tid < TW) wsreg[d] = load_scale_dw(wsptr, blk0);
+            if (tid < TM) asreg[d] = load_scale_dw(asptr, blk0);
+        }
+    };
+    auto store_lds = [&](uint32_t stage) {
+        uint8_t* sW = smem + stage * kStageBytes;
+        uint8_t* sA = sW + TW * kSlabBytes;
+        uint32_t* sWs = reinterpret_cast<uint32_t*>(sA + TM * kSlabBytes);
+        uint32_t* sAs = sWs + TW * kScaleDw;
+#pragma unroll
+        for (int j = 0; j < kWLoads; ++j) {
+            const uint32_t r = ld_row + 32 * j;
+            *reinterpret_cast<uint4*>(sW + r * kSlabBytes + swz(r, ld_chunk) * 16) = wreg[j];
+        }
+#pragma unroll
+        for (int j = 0; j < kALoads; ++j) {
+            const uint32_t r = ld_row + 32 * j;
+            *reinterpret_cast<uint4*>(sA + r * kSlabBytes + swz(r, ld_chunk) * 16) = areg[j];
+        }
+#pragma unroll
+        for (int d = 0; d < kScaleDw; ++d) {
+            if (tid < TW) sWs[tid * kScaleDw + d] = wsreg[d];
+            if (tid < TM) sAs[tid * kScaleDw + d] = asreg[d];
+        }
+    };
+
+    // ---- accumulators --------------------------------------------------------------------------
+    v16f acc[FW][FM];
+#pragma unroll
+    for (int i = 0; i < FW; ++i)
+#pragma unroll
+        for (int j = 0; j < FM; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+
+    // LDS row of the wavefront's fragment f
+    auto wfrag_row = [&](int f) -> uint32_t {
+        if (EPI == kEpiSwigluQuant)
+            return f < FW / 2 ? ww * (TW / 2 / WW) + f * 32 : TW / 2 + ww * (TW / 2 / WW) + (f - FW / 2) * 32;
+        return ww * (TW / WW) + f * 32;
+    };
+    const uint32_t l32 = lane & 31u, lh = lane >> 5;
+
+    auto compute = [&](uint32_t stage) {
+        const uint8_t* sW = smem + stage * kStageBytes;
+        const uint8_t* sA = sW + TW * kSlabBytes;
+        const uint32_t* sWs = reinterpret_cast<const uint32_t*>(sA + TM * kSlabBytes);
+        const uint32_t* sAs = sWs + TW * kScaleDw;
+        // lane's scale registers: byte 2*h' (after the lh shift) belongs to MFMA step h' of the dword
+        uint32_t sw[FW][kScaleDw], sa[FM][kScaleDw];
+#pragma unroll
+        for (int f = 0; f < FW; ++f)
+#pragma unroll
+            for (int d = 0; d < kScaleDw; ++d) sw[f][d] = sWs[(wfrag_row(f) + l32) * kScaleDw + d] >> (8 * lh);
+#pragma unroll
+        for (int f = 0; f < FM; ++f)
+#pragma unroll
+            for (int d = 0; d < kScaleDw; ++d)
+                sa[f][d] = sAs[(wm * (TM / WM) + f * 32 + l32) * kScaleDw + d] >> (8 * lh);
+
+#pragma unroll
+        for (int h = 0; h < kSub; ++h) {
+            v8i af[FM];
+#pragma unroll
+            for (int f = 0; f < FM; ++f) {
+                const uint32_t r = wm * (TM / WM) + f * 32 + l32;
+                const uint8_t* rp = sA + r * kSlabBytes;
+                if (kFp4) {
+                    const uint32_t c0 = h * 2 + lh;
+                    v4i lo = *reinterpret_cast<const v4i*>(rp + swz(r, c0) * 16);
+                    af[f] = (v8i){lo[0], lo[1], lo[2], lo[3], 0, 0, 0, 0};
+                } else {
+                    // 8-bit operands: registers 0-3 carry k = 16*lh + [0,16) of the step's first
+                    // 32-block, registers 4-7 the same slice of its second 32-block
+                    const uint32_t c0 = h * 4 + lh;
+                    v4i lo = *reinterpret_cast<const v4i*>(rp + swz(r, c0) * 16);
+                    v4i hi = *reinterpret_cast<const v4i*>(rp + swz(r, c0 + 2) * 16);
+                    af[f] = (v8i){lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+                }
+            }
+#pragma unroll
+            for (int fw = 0; fw < FW; ++fw) {
+                const uint32_t r = wfrag_row(fw) + l32;
+                const uint8_t* rp = sW + r * kSlabBytes;
+                v8i wf;
+                if (kFp4) {
+                    const uint32_t c0 = h * 2 + lh;
+                    v4i lo = *reinterpret_cast<const v4i*>(rp + swz(r, c0) * 16);
+                    wf = (v8i){lo[0], lo[1], lo[2], lo[3], 0, 0, 0, 0};
+                } else {
+                    const uint32_t c0 = h * 4 + lh;
+                    v4i lo = *reinterpret_cast<const v4i*>(rp + swz(r, c0) * 16);
+                    v4i hi = *reinterpret_cast<const v4i*>(rp + swz(r, c0 + 2) * 16);
+                    wf = (v8i){lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+                }
+#pragma unroll
+                for (int fm = 0; fm < FM; ++fm) {
+                    // step h uses scale dword h/2, byte 2*(h%2) of the shifted register
+                    acc[fw][fm] = mfma<FMT>(wf, af[fm], acc[fw][fm], (h & 1) * 2, (int)sw[fw][h >> 1],
+                                            (int)sa[fm][h >> 1]);
+                }
+            }
+        }
+    };
+
+    // ---- main loop -------------------------------------------------------------------------------
+    load_global(0);
+    store_lds(0);
+    __syncthreads();
+    for (uint32_t s = 0; s < nslab; ++s) {
+        const bool more = s + 1 < nslab;
+        if (more) load_global(s + 1);
+        compute(s & 1u);
+        if (more) store_lds((s + 1) & 1u);
+        __syncthreads();
+    }
+
+    // ---- epilogue ----------------------------------------------------------------------------------
+    if constexpr (EPI == kEpiStore) {
+#pragma unroll
+        for (int fm = 0; fm < FM; ++fm) {
+            const uint32_t mloc = wm * (TM / WM) + fm * 32 + l32;
+            if (mloc >= rows_valid) continue;
+            const size_t mrow = (size_t)(row0 + mloc);
+#pragma unroll
+            for (int fw = 0; fw < FW; ++fw) {
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    const uint32_t ncol = wt * TW + wfrag_row(fw) + 8 * q + 4 * lh;
+                    if (ncol >= p.n) continue;
+                    const v4f v = to_v4(acc[fw][fm], q);
+                    const bool full = ncol + 4 <= p.n;
+                    if (p.out_type == CMX_OUT_BF16) {
+                        uint16_t* o = reinterpret_cast<uint16_t*>(p.c) + mrow * p.ldc + ncol;
+                        uint32_t b0 = f32_to_bf16(v[0]), b1 = f32_to_bf16(v[1]), b2 = f32_to_bf16(v[2]),
+                                 b3 = f32_to_bf16(v[3]);
+                        if (full && (p.ldc % 4 == 0)) {
+                            *reinterpret_cast<uint2*>(o) = make_uint2(b0 | (b1 << 16), b2 | (b3 << 16));
+                        } else {
+                            uint32_t bb[4] = {b0, b1, b2, b3};
+                            for (uint32_t i = 0; i < 4 && ncol + i < p.n; ++i) o[i] = (uint16_t)bb[i];
+                        }
+                    } else if (p.out_type == CMX_OUT_FP16) {
+                        _Float16* o = reinterpret_cast<_Float16*>(p.c) + mrow * p.ldc + ncol;
+                        for (uint32_t i = 0; i < 4 && ncol + i < p.n; ++i) o[i] = (_Float16)v[i];
+                    } else {
+                        float* o = reinterpret_cast<float*>(p.c) + mrow * p.ldc + ncol;
+                        for (uint32_t i = 0; i < 4 && ncol + i < p.n; ++i) o[i] = v[i];
+                    }
+                }
+            }
+        }
+    } else {
+        const uint32_t half = p.n >> 1;
+#pragma unroll
+        for (int fm = 0; fm < FM; ++fm) {
+            const uint32_t mloc = wm * (TM / WM) + fm * 32 + l32;
+            const bool mvalid = mloc < rows_valid;
+            const size_t mrow = (size_t)(row0 + (mvalid ? mloc : 0));
+#pragma unroll
+            for (int f = 0; f < FW / 2; ++f) {
+                // activation column of this fragment's 32-wide MX block
+                const uint32_t ncol0 = wt * (TW / 2) + ww * (TW / 2 / WW) + f * 32;
+                float actv[16];
+                uint32_t amax = 0;
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const float hg = bf16_to_f32(f32_to_bf16(acc[f][fm][r]));
+                    const float hu = bf16_to_f32(f32_to_bf16(acc[f + FW / 2][fm][r]));
+                    const uint32_t ab = f32_to_bf16(silu_mul(hg, hu));
+                    actv[r] = bf16_to_f32(ab);
+                    const uint32_t mag = ab & 0x7FFFu;
+                    amax = amax > mag ? amax : mag;
+                    if (p.act_bf16 && mvalid) {
+                        const uint32_t ncol = ncol0 + 8 * (r >> 2) + 4 * lh + (r & 3);
+                        if (ncol < half) p.act_bf16[mrow * half + ncol] = (uint16_t)ab;
+                    }
+                }
+                const uint32_t other = (uint32_t)__shfl_xor((int)amax, 32);
+                amax = amax > other ? amax : other;
+                const int e = block_exp_from_bf16_amax(amax, kEmaxE4M3);
+                if (!mvalid || ncol0 >= half) continue;
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    float y0 = clamp_abs(ldexpf(actv[4 * q + 0], -e), 448.0f);
+                    float y1 = clamp_abs(ldexpf(actv[4 * q + 1], -e), 448.0f);
+                    float y2 = clamp_abs(ldexpf(actv[4 * q + 2], -e), 448.0f);
+                    float y3 = clamp_abs(ldexpf(actv[4 * q + 3], -e), 448.0f);
+                    uint32_t wv = cvt_pk_e4m3(y0, y1, 0u, false);
+                    wv = cvt_pk_e4m3(y2, y3, wv, true);
+                    *reinterpret_cast<uint32_t*>(p.act_codes + mrow * p.ld_act + ncol0 + 8 * q + 4 * lh) = wv;
+                }
+                if (lh == 0) {
+                    uint8_t* srow = p.act_scales + mrow * p.ld_acts;
+                    const uint32_t blk = ncol0 >> 5;
+                    srow[blk] = (uint8_t)(e + 127);
+                    const uint32_t nblk = half >> 5;
+                    if (blk == nblk - 1 && (nblk & 1u)) srow[nblk] = 127;
+                }
+            }
+        }
+    }
+}
+
+// Row offsets and m-tile prefix of the groups (one workgroup).
+__global__ void gmm_prepare_kernel(const int32_t* __restrict__ sizes, uint32_t groups, uint32_t tile_m,
+                                   int32_t* __restrict__ row_off, int32_t* __restrict__ tile_pref) {
+    extern __shared__ int32_t sh[];
+    for (uint32_t i = threadIdx.x; i < groups; i += blockDim.x) sh[i] = sizes[i] > 0 ? sizes[i] : 0;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        int32_t r = 0, t = 0;
+        for (uint32_t i = 0; i < groups; ++i) {
+            row_off[i] = r;
+            tile_pref[i] = t;
+            r += sh[i];
+            t += (sh[i] + (int32_t)tile_m - 1) / (int32_t)tile_m;
+        }
+        row_off[groups] = r;
+        tile_pref[groups] = t;
+    }
+}
+
+template <int FMT, int TW, int TM, int WW, int WM, int EPI>
+int launch_gemm(const GemmParams& p, uint32_t max_m_tiles, hipStream_t s) {
+    constexpr int kScaleDw = FMT == CMX_FMT_E2M1 ? 2 : 1;
+    constexpr size_t smem = 2 * ((TW + TM) * kSlabBytes + (TW + TM) * 4 * kScaleDw);
+    auto kfn = mx_gemm_kernel<FMT, TW, TM, WW, WM, EPI>;
+    static bool attr_set = false;
+    if (!attr_set) {
+        CMX_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kfn), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                    (int)smem));
+        attr_set = true;
+    }
+    const uint64_t tiles = (uint64_t)max_m_tiles * p.w_tiles;
+    CMX_REQUIRE(tiles > 0 && tiles < (1ull << 31), "tile count out of range");
+    hipLaunchKernelGGL(kfn, dim3((uint32_t)tiles), dim3(kThreads), smem, s, p);
+    CMX_LAUNCH_CHECK();
+    return CMX_OK;
+}
+
+struct TileChoice {
+    int tw, tm;
+};
+
+int g_force_tile = 0;   // test/tuning hook: 0 = heuristic, else tw*1000 + tm
+
+TileChoice choose_tile(uint32_t m_hint, uint32_t n) {
+    if (g_force_tile) return {g_force_tile / 1000, g_force_tile % 1000};
+    if (m_hint <= 64) return {256, 64};
+    if (m_hint <= 128) return {256, 128};
+    return {256, 256};
+}
+
+template <int FMT, int EPI>
+int dispatch_tile(const GemmParams& p, TileChoice t, uint32_t max_m_tiles, hipStream_t s) {
+    if (t.tw == 256 && t.tm == 256) return launch_gemm<FMT, 256, 256, 2, 2, EPI>(p, max_m_tiles, s);
+    if (t.tw == 256 && t.tm == 128) return launch_gemm<FMT, 256, 128, 2, 2, EPI>(p, max_m_tiles, s);
+    if (t.tw == 256 && t.tm == 64) return launch_gemm<FMT, 256, 64, 4, 1, EPI>(p, max_m_tiles, s);
+    if (t.tw == 128 && t.tm == 128) return launch_gemm<FMT, 128, 128, 2, 2, EPI>(p, max_m_tiles, s);
+    set_error("unsupported tile shape");
+    return CMX_EINVAL;
+}
+
+int check_operands(const void* a, uint32_t lda, const void* as, uint32_t ld_as, const void* w, uint32_t ldw,
+                   const void* ws, uint32_t ld_ws, uint32_t k, int fmt) {
+    CMX_REQUIRE(a && as && w && ws, "null pointer");
+    CMX_REQUIRE(fmt == CMX_FMT_E4M3 || fmt == CMX_FMT_E5M2 || fmt == CMX_FMT_E2M1, "unknown element format");
+    CMX_REQUIRE(k > 0 && k % 32 == 0, "k must be a positive multiple of 32");
+    const uint32_t kbytes = fmt == CMX_FMT_E2M1 ? k / 2 : k;
+    CMX_REQUIRE(lda >= kbytes && ldw >= kbytes, "operand row pitch smaller than a row");
+    CMX_REQUIRE(lda % 16 == 0 && ldw % 16 == 0 && aligned16(a) && aligned16(w), "operand rows must be 16-byte aligned");
+    CMX_REQUIRE(ld_as >= k / 32 && ld_ws >= k / 32, "scale row pitch smaller than a row");
+    return CMX_OK;
+}
+
+bool scales_dword_aligned(const void* as, uint32_t ld_as, const void* ws, uint32_t ld_ws) {
+    return ld_as % 4 == 0 && ld_ws % 4 == 0 && (reinterpret_cast<uintptr_t>(as) & 3u) == 0 &&
+           (reinterpret_cast<uintptr_t>(ws) & 3u) == 0;
+}
+
+}  // namespace
+
+}  // namespace cmx
+
+extern "C" int cmx_debug_force_tile(int tw, int tm) {
+    cmx::g_force_tile = (tw > 0 && tm > 0) ? tw * 1000 + tm : 0;
+    return CMX_OK;
+}
+
+extern "C" int cmx_mx_gemm(const uint8_t* a, uint32_t lda, const uint8_t* a_scale, uint32_t ld_as, const uint8_t* b,
+                           uint32_t ldb, const uint8_t* b_scale, uint32_t ld_bs, void* c, uint32_t ldc, uint32_t m,
+                           uint32_t n, uint32_t k, int fmt, int out_type, cmx_stream_t stream) {
+    using namespace cmx;
+    if (m == 0 || n == 0) return CMX_OK;
+    int rc = check_operands(a, lda, a_scale, ld_as, b, ldb, b_scale, ld_bs, k, fmt);
+    if (rc != CMX_OK) return rc;
+    CMX_REQUIRE(c && ldc >= n, "bad output");
+    CMX_REQUIRE(out_type == CMX_OUT_BF16 || out_type == CMX_OUT_FP16 || out_type == CMX_OUT_FP32, "unknown output type");
+    GemmParams p{};
+    p.a = a; p.a_scale = a_scale; p.w = b; p.w_scale = b_scale; p.c = c;
+    p.lda = lda; p.ld_as = ld_as; p.ldw = ldb; p.ld_ws = ld_bs; p.ldc = ldc;
+    p.m = m; p.n = n; p.kbytes = fmt == CMX_FMT_E2M1 ? k / 2 : k; p.kblocks = k / 32;
+    p.groups = 1; p.out_type = out_type;
+    p.scale_vec = scales_dword_aligned(a_scale, ld_as, b_scale, ld_bs);
+    TileChoice t = choose_tile(m, n);
+    p.w_tiles = ceil_div(n, t.tw);
+    const uint32_t m_tiles = ceil_div(m, t.tm);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    switch (fmt) {
+        case CMX_FMT_E4M3: return dispatch_tile<CMX_FMT_E4M3, kEpiStore>(p, t, m_tiles, s);
+        case CMX_FMT_E5M2: return dispatch_tile<CMX_FMT_E5M2, kEpiStore>(p, t, m_tiles, s);
+        default: return dispatch_tile<CMX_FMT_E2M1, kEpiStore>(p, t, m_tiles, s);
+    }
+}
+
+extern "C" size_t cmx_mx_gmm_workspace_bytes(uint32_t groups) {
+    return cmx::round_up_sz(2 * (size_t)(groups + 1) * sizeof(int32_t), 256);
+}
+
+namespace cmx {
+namespace {
+int gmm_common(GemmParams& p, const int32_t* group_sizes, uint32_t groups, uint32_t m_total, void* workspace, int fmt,
+               bool swiglu, hipStream_t s) {
+    CMX_REQUIRE(group_sizes && workspace, "null pointer");
+    CMX_REQUIRE(groups > 0 && groups <= 65536, "bad group count");
+    CMX_REQUIRE((reinterpret_cast<uintptr_t>(workspace) & 3u) == 0, "workspace must be 4-byte aligned");
+    // average rows per group steers the tile height
+    TileChoice t = choose_tile(ceil_div(m_total, groups), p.n);
+    int32_t* row_off = static_cast<int32_t*>(workspace);
+    int32_t* tile_pref = row_off + (groups + 1);
+    hipLaunchKernelGGL(gmm_prepare_kernel, dim3(1), dim3(256), groups * sizeof(int32_t), s, group_sizes, groups,
+                       (uint32_t)t.tm, row_off, tile_pref);
+    CMX_LAUNCH_CHECK();
+    p.row_off = row_off;
+    p.tile_pref = tile_pref;
+    p.groups = groups;
+    p.w_tiles = swiglu ? ceil_div(p.n / 2, t.tw / 2) : ceil_div(p.n, t.tw);
+    const uint32_t max_m_tiles = m_total / t.tm + groups;
+    if (swiglu) return dispatch_tile<CMX_FMT_E4M3, kEpiSwigluQuant>(p, t, max_m_tiles, s);
+    switch (fmt) {
+        case CMX_FMT_E4M3: return dispatch_tile<CMX_FMT_E4M3, kEpiStore>(p, t, max_m_tiles, s);
+        case CMX_FMT_E5M2: return dispatch_tile<CMX_FMT_E5M2, kEpiStore>(p, t, max_m_tiles, s);
+        default: return dispatch_tile<CMX_FMT_E2M1, kEpiStore>(p, t, max_m_tiles, s);
+    }
+}
+}  // namespace
+}  // namespace cmx
+
+extern "C" int cmx_mx_gmm(const uint8_t* a, uint32_t lda, const uint8_t* a_scale, uint32_t ld_as, const uint8_t* b,
+                          const uint8_t* b_scale, void* c, uint32_t ldc, const int32_t* group_sizes, uint32_t groups,
+                          uint32_t m_total, uint32_t n, uint32_t k, int fmt, int out_type, void* workspace,
+                          cmx_stream_t stream) {
+    using namespace cmx;
+    if (m_total == 0 || n == 0) return CMX_OK;
+    const uint32_t kbytes = fmt == CMX_FMT_E2M1 ? k / 2 : k;
+    int rc = check_operands(a, lda, a_scale, ld_as, b, kbytes, b_scale, k / 32, k, fmt);
+    if (rc != CMX_OK) return rc;
+    CMX_REQUIRE(c && ldc >= n, "bad output");
+    CMX_REQUIRE(out_type == CMX_OUT_BF16 || out_type == CMX_OUT_FP16 || out_type == CMX_OUT_FP32, "unknown output type");
+    GemmParams p{};
+    p.a = a; p.a_scale = a_scale; p.w = b; p.w_scale = b_scale; p.c = c;
+    p.lda = lda; p.ld_as = ld_as; p.ldw = kbytes; p.ld_ws = k / 32; p.ldc = ldc;
+    p.m = m_total; p.n = n; p.kbytes = kbytes; p.kblocks = k / 32; p.out_type = out_type;
+    p.scale_vec = scales_dword_aligned(a_scale, ld_as, b_scale, k / 32);
+    return gmm_common(p, group_sizes, groups, m_total, workspace, fmt, false, static_cast<hipStream_t>(stream));
+}
+
+extern "C" int cmx_mx_gmm_swiglu_quant(const uint8_t* a, uint32_t lda, const uint8_t* a_scale, uint32_t ld_as,
+                                       const uint8_t* b, const uint8_t* b_scale, uint8_t* act_codes, uint32_t ld_act,
+                                       uint8_t* act_scales, uint32_t ld_acts, void* act_bf16,
+                                       const int32_t* group_sizes, uint32_t groups, uint32_t m_total, uint32_t n,
+                                       uint32_t k, void* workspace, cmx_stream_t stream) {
+    using namespace cmx;
+    if (m_total == 0 || n == 0) return CMX_OK;
+    int rc = check_operands(a, lda, a_scale, ld_as, b, k, b_scale, k / 32, k, CMX_FMT_E4M3);
+    if (rc != CMX_OK) return rc;
+    CMX_REQUIRE(n % 64 == 0, "n must be a multiple of 64 (gate|up halves of whole MX blocks)");
+    CMX_REQUIRE(act_codes && act_scales, "null pointer");
+    CMX_REQUIRE(ld_act >= n / 2 && ld_act % 4 == 0 && (reinterpret_cast<uintptr_t>(act_codes) & 3u) == 0,
+                "activation code rows must be 4-byte aligned and hold n/2 bytes");
+    CMX_REQUIRE(ld_acts >= scale_cols(n / 2), "activation scale pitch too small");
+    GemmParams p{};
+    p.a = a; p.a_scale = a_scale; p.w = b; p.w_scale = b_scale;
+    p.act_codes = act_codes; p.act_scales = act_scales; p.act_bf16 = static_cast<uint16_t*>(act_bf16);
+    p.ld_act = ld_act; p.ld_acts = ld_acts;
+    p.lda = lda; p.ld_as = ld_as; p.ldw = k; p.ld_ws = k / 32;
+    p.m = m_total; p.n = n; p.kbytes = k; p.kblocks = k / 32; p.out_type = CMX_OUT_BF16;
+    p.scale_vec = scales_dword_aligned(a_scale, ld_as, b_scale, k / 32);
+    return gmm_common(p, group_sizes, groups, m_total, workspace, CMX_FMT_E4M3, true, static_cast<hipStream_t>(stream));
+}

@@ -1,0 +1,229 @@
+/*
+ * catccos_mx.h - C ABI of the MI355X (gfx950) MX compute core.
+ *
+ * Plain C: pointers are device pointers unless a parameter is named host_*, sizes are in
+ * elements unless a name ends in _bytes.  Every entry point is asynchronous on `stream`
+ * (a hipStream_t passed as void*; NULL = the default stream) and returns 0 on success or a
+ * negative CMX_E* code; cmx_last_error() returns a thread-local message for the last
+ * failure.  Nothing here allocates device memory except the cmx_rt_* runtime shim.
+ *
+ * Each group names the reference interface it replaces (paths relative to the reference
+ * checkout).
+ */
+#ifndef CATCCOS_MX_H
+#define CATCCOS_MX_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define CMX_OK 0
+#define CMX_EINVAL (-1)   /* bad argument (shape, alignment, null pointer) */
+#define CMX_ERUNTIME (-2) /* HIP runtime reported an error               */
+#define CMX_ENOSPACE (-3) /* workspace too small                         */
+
+/* element formats (E8M0 block-32 scales in every case) */
+#define CMX_FMT_E4M3 0
+#define CMX_FMT_E5M2 1
+#define CMX_FMT_E2M1 2 /* FP4, two codes per byte, even column in the low nibble */
+
+/* rounding of the element cast */
+#define CMX_ROUND_RNE 0 /* IEEE nearest-even: runtime activations            */
+#define CMX_ROUND_LUT 1 /* nearest table value, tie -> smaller magnitude, -0 -> +0: offline weights, FP4 golden */
+
+/* output types of the matmul entry points */
+#define CMX_OUT_BF16 0
+#define CMX_OUT_FP16 1
+#define CMX_OUT_FP32 2
+
+typedef void* cmx_stream_t;
+
+int cmx_version(void);
+const char* cmx_last_error(void);
+
+/* ------------------------------------------------------------------------------------------
+ * Runtime shim: what the host plugin layer needs from the device runtime.
+ * Replaces aclrtMalloc / aclrtFree / aclrtMallocHost / aclrtFreeHost / aclrtMemcpy /
+ * aclrtMemset / aclrtSynchronizeStream as used by utils/info.h:134-214 and every
+ * examples/<op>/<op>_host.h AllocateDeviceSpace / WriteResultFile.
+ * ---------------------------------------------------------------------------------------- */
+int cmx_rt_device_count(int* count);
+int cmx_rt_set_device(int device);
+int cmx_rt_malloc(void** ptr, size_t bytes);
+int cmx_rt_free(void* ptr);
+int cmx_rt_malloc_host(void** ptr, size_t bytes);
+int cmx_rt_free_host(void* ptr);
+int cmx_rt_memcpy_h2d(void* dst, const void* host_src, size_t bytes);
+int cmx_rt_memcpy_d2h(void* host_dst, const void* src, size_t bytes);
+int cmx_rt_memset(void* dst, int value, size_t bytes);
+int cmx_rt_stream_create(cmx_stream_t* stream);
+int cmx_rt_stream_destroy(cmx_stream_t stream);
+int cmx_rt_stream_sync(cmx_stream_t stream);
+
+/* ------------------------------------------------------------------------------------------
+ * MX block quantizer.
+ * Replaces CommBlockMxQuant::operator() / ComputeMxQuant
+ * (include/catccos/comm/block/comm_block_mx_quant.hpp:154-316, 412-664) launched by
+ * MxQuantAllGather<<<>>> (examples/ascend950_mx_quant_allgather/mx_quant_allgather_device.h:108-141);
+ * results follow the golden _quantize_axis_last_fp8 / _quantize_axis_last
+ * (examples/utils/gen_mx_quant_allgather_data.py:255-313, 414-449).
+ *
+ *   x       bf16 [rows, cols], row pitch ld_x elements
+ *   codes   u8   [rows, cols] (FP4: [rows, ceil(cols/2)]), row pitch ld_codes bytes
+ *   scales  u8   [rows, RoundUp2(ceil(cols/32))], row pitch ld_scales bytes; padding column = 127
+ * ---------------------------------------------------------------------------------------- */
+int cmx_mx_quant(const void* x, uint32_t ld_x, uint8_t* codes, uint32_t ld_codes, uint8_t* scales,
+                 uint32_t ld_scales, uint32_t rows, uint32_t cols, int fmt, int round_mode, cmx_stream_t stream);
+
+/* Dequantize (test/debug helper, same layouts): out fp32 [rows, cols]. */
+int cmx_mx_dequant(const uint8_t* codes, uint32_t ld_codes, const uint8_t* scales, uint32_t ld_scales, float* out,
+                   uint32_t ld_out, uint32_t rows, uint32_t cols, int fmt, cmx_stream_t stream);
+
+/* ------------------------------------------------------------------------------------------
+ * Dense MX matmul  C[m,n] = sum_k deq(A)[m,k] * deq(B)[n,k]   (both operands K-contiguous).
+ * Replaces the AIC loop of MatmulReduceScatterMxTla
+ * (include/catccos/dgemm/kernel/matmul_reduce_scatter_mx_tla.hpp:190-315: blockMmad(A,B,C,shape,
+ * scaleA,scaleB)) for one device's full M x N x K product; golden
+ * examples/ascend950_mxfp8_matmul_reduce_scatter/scripts/gen_data_mxfp8_mmrs.py:343-355.
+ *
+ *   a  codes [m, k] (FP4: k/2 bytes), pitch lda bytes;  a_scale u8 [m, k/32], pitch ld_as bytes
+ *   b  codes [n, k] (transposed weight), pitch ldb;     b_scale u8 [n, k/32], pitch ld_bs
+ *   c  [m, n] of out_type, pitch ldc elements
+ * k must be a multiple of 32; operand rows 16-byte aligned.
+ * ---------------------------------------------------------------------------------------- */
+int cmx_mx_gemm(const uint8_t* a, uint32_t lda, const uint8_t* a_scale, uint32_t ld_as, const uint8_t* b,
+                uint32_t ldb, const uint8_t* b_scale, uint32_t ld_bs, void* c, uint32_t ldc, uint32_t m,
+                uint32_t n, uint32_t k, int fmt, int out_type, cmx_stream_t stream);
+
+/* ------------------------------------------------------------------------------------------
+ * Grouped MX matmul over ragged expert groups.
+ * Replaces the AIC tile loops of Ascend950GmmAllToAllKernel
+ * (include/catccos/dgemm/kernel/ascend950_gmm_alltoall.hpp:219-324) and
+ * MxAllToAllVGroupedMatmulTla (include/catccos/dgemm/kernel/mx_alltoallv_group_matmul.hpp),
+ * including their per-expert offset arithmetic (ascend950_alltoall_gmm.hpp:238-322).
+ *
+ *   group_sizes  int32 [groups] ON DEVICE (rows per expert, in order; zeros allowed)
+ *   a / a_scale  rows of all groups back to back, m_total = sum(group_sizes) rows
+ *   b / b_scale  [groups, n, k] / [groups, n, k/32], dense
+ *   c            [m_total, n]
+ *   workspace    >= cmx_mx_gmm_workspace_bytes(groups) bytes (tile schedule metadata)
+ * Rows beyond sum(group_sizes) (up to m_total) are left untouched.
+ * ---------------------------------------------------------------------------------------- */
+size_t cmx_mx_gmm_workspace_bytes(uint32_t groups);
+int cmx_mx_gmm(const uint8_t* a, uint32_t lda, const uint8_t* a_scale, uint32_t ld_as, const uint8_t* b,
+               const uint8_t* b_scale, void* c, uint32_t ldc, const int32_t* group_sizes, uint32_t groups,
+               uint32_t m_total, uint32_t n, uint32_t k, int fmt, int out_type, void* workspace,
+               cmx_stream_t stream);
+
+/* ------------------------------------------------------------------------------------------
+ * Grouped MXFP8 matmul with fused SwiGLU and MX requant (GMM1 of the FFN).
+ * Replaces Ascend950AllToAllGmmKernel's AIC loop (ascend950_alltoall_gmm.hpp:193-323: gate and
+ * up products per tile) + SwigluBf16RegBaseVf
+ * (include/catccos/epilogue/block/block_epilogue_regbase_swiglu.hpp:38-78) +
+ * Ascend950SwigluMxQuantFromUbKernel::ComputeUbTile
+ * (examples/aux_ops/ascend950_swiglu_from_ub.h:333-373); golden gen_data_moe.py:646-658.
+ *
+ *   b / b_scale   [groups, n, k]: rows [0, n/2) = gate (gets SiLU), rows [n/2, n) = up
+ *   act_codes     u8 E4M3 [m_total, n/2], pitch ld_act bytes
+ *   act_scales    u8 E8M0 [m_total, RoundUp2(n/64)], pitch ld_acts bytes
+ *   act_bf16      optional (may be NULL): bf16 [m_total, n/2] SwiGLU output before requant
+ * n must be a multiple of 64.  h = bf16(A.B) and act = bf16(silu(gate)*up) are both rounded to
+ * bf16 before the next step, as the golden does.
+ * ---------------------------------------------------------------------------------------- */
+int cmx_mx_gmm_swiglu_quant(const uint8_t* a, uint32_t lda, const uint8_t* a_scale, uint32_t ld_as,
+                            const uint8_t* b, const uint8_t* b_scale, uint8_t* act_codes, uint32_t ld_act,
+                            uint8_t* act_scales, uint32_t ld_acts, void* act_bf16, const int32_t* group_sizes,
+                            uint32_t groups, uint32_t m_total, uint32_t n, uint32_t k, void* workspace,
+                            cmx_stream_t stream);
+
+/* ------------------------------------------------------------------------------------------
+ * MoE routing: stable sort of (expert, row) pairs.
+ * Replaces moe_init_routing_v2 (examples/aux_ops/moe_init_routing_v2/moe_init_routing_v2.h:56-220,
+ * moe_v2_src_to_dst_op_simt.h:79-87); golden moe_init_routing_cpu (gen_data_moe.py:48-57).
+ *
+ *   expert_idx   int32 [tokens, top_k], values in [0, experts)
+ *   sorted2src   int32 [tokens*top_k]  = stable argsort of the flattened ids (golden direction)
+ *   src2sorted   int32 [tokens*top_k]  = inverse (the device's expandedRowIdx)
+ *   counts       int32 [experts]       = rows per expert
+ *   workspace    >= cmx_moe_routing_workspace_bytes(tokens*top_k, experts)
+ * ---------------------------------------------------------------------------------------- */
+size_t cmx_moe_routing_workspace_bytes(uint32_t routes, uint32_t experts);
+int cmx_moe_init_routing(const int32_t* expert_idx, uint32_t tokens, uint32_t top_k, uint32_t experts,
+                         int32_t* sorted2src, int32_t* src2sorted, int32_t* counts, void* workspace,
+                         cmx_stream_t stream);
+
+/* ------------------------------------------------------------------------------------------
+ * Fused dispatch on one device: quantize each token once (E4M3, RNE) and write the row to its
+ * top_k destinations.  Replaces CommBlockMxQuant::QuantScatterPacked
+ * (comm_block_mx_quant.hpp:318-368) via QuantScatterRoutingMxFp8
+ * (examples/ascend950_dispatch_ffn_combine/ascend950_dispatch_ffn_combine_device.h:611-644).
+ *
+ *   x           bf16 [tokens, k]
+ *   src2sorted  int32 [tokens*top_k]; negative destinations are skipped
+ *   out_codes   row r at out_codes + r*ld_out;  out_scales row r at out_scales + r*ld_outs
+ * The reference's packed wire row [codes k | scales RoundUp2(k/32) | pad to 32 B] is the case
+ * out_scales = out_codes + k, ld_out = ld_outs = cmx_packed_row_bytes(k).
+ * ---------------------------------------------------------------------------------------- */
+uint32_t cmx_packed_row_bytes(uint32_t k);
+int cmx_quant_scatter(const void* x, uint32_t ld_x, const int32_t* src2sorted, uint8_t* out_codes, uint32_t ld_out,
+                      uint8_t* out_scales, uint32_t ld_outs, uint32_t tokens, uint32_t k, uint32_t top_k,
+                      cmx_stream_t stream);
+
+/* ------------------------------------------------------------------------------------------
+ * Weighted top-k combine.  Replaces KernelMoeTokenUnpermute<bf16,int32,float,true>
+ * (examples/aux_ops/moe_token_unpermute/moe_token_unpermute.h:233-366):
+ * out[t] = bf16( sum_k probs[t,k] * y[src2sorted[t*top_k+k]] ), fp32 multiply then fp32 add in k
+ * order; indices outside [0, rows) contribute nothing.
+ * ---------------------------------------------------------------------------------------- */
+int cmx_moe_token_unpermute(const void* y, uint32_t ld_y, uint32_t rows, const int32_t* src2sorted,
+                            const float* probs, void* out, uint32_t ld_out, uint32_t tokens, uint32_t hidden,
+                            uint32_t top_k, cmx_stream_t stream);
+
+/* ------------------------------------------------------------------------------------------
+ * Full single-device MoE FFN: dispatch -> GMM1 -> SwiGLU -> requant -> GMM2 -> combine.
+ * Same argument list as CatccosKernel::catccos_ascend950_dispatch_ffn_combine_wrapper
+ * (examples/torch_binding/include/catccos_torch_kernel.h:40-44, body
+ * examples/ascend950_dispatch_ffn_combine/ascend950_dispatch_ffn_combine_wrapper.cpp:18-66) and
+ * catccos_ascend950_symmetric_bytes (:24).  blockDim, fftsAddr and symmetric are accepted and
+ * ignored (no cube/vector split and no peers on one GPU); rankSize must be 1.
+ *
+ *   x bf16 [m,k]; expertIdx int32 [m,topK]; gateWeight fp32 [m,topK]
+ *   w1 E4M3 [E,n,k], w1Scale [E,n,k/32]; w2 [E,k,n/2], w2Scale [E,k,n/64]; out bf16 [m,k]
+ *   workspace >= catccos_ascend950_dispatch_ffn_combine_workspace_bytes(...) ; contents may be
+ *   garbage on entry.
+ * ---------------------------------------------------------------------------------------- */
+uint64_t catccos_ascend950_symmetric_bytes(void);
+size_t catccos_ascend950_dispatch_ffn_combine_workspace_bytes(uint32_t m, uint32_t k, uint32_t n,
+                                                              uint32_t localExperts, uint32_t topK, int rankSize);
+int catccos_ascend950_dispatch_ffn_combine(uint32_t blockDim, cmx_stream_t stream, uint64_t fftsAddr,
+                                           const uint8_t* x, const uint8_t* expertIdx, const uint8_t* gateWeight,
+                                           const uint8_t* w1, const uint8_t* w1Scale, const uint8_t* w2,
+                                           const uint8_t* w2Scale, uint8_t* out, uint8_t* workspace,
+                                           uint8_t* symmetric, uint32_t m, uint32_t k, uint32_t n,
+                                           uint32_t localExperts, uint32_t topK, int rankSize);
+
+/* Offsets of the FFN's intermediate buffers inside the workspace (for tests and debugging). */
+typedef struct cmx_ffn_workspace_layout {
+    size_t src2sorted, sorted2src, counts, routing_scratch, gmm_meta;
+    size_t a_codes, a_scales, act_codes, act_scales, y;
+    size_t total;
+} cmx_ffn_workspace_layout;
+int cmx_ffn_workspace_layout_get(uint32_t m, uint32_t k, uint32_t n, uint32_t localExperts, uint32_t topK,
+                                 cmx_ffn_workspace_layout* layout);
+
+/* ------------------------------------------------------------------------------------------
+ * Single-tile probe of the block-scaled MFMA (used by the layout known-answer tests):
+ * out fp32 [32, 32] = deq(w)[32 rows, 64 k] . deq(a)[32 rows, 64 k]^T with one E8M0 scale per
+ * (row, 32-k block).  w/a: fmt codes [32, 64] (FP4: [32, 32] bytes); ws/as: u8 [32, 2].
+ * out[i][j] = sum_k w[i,k] * a[j,k].
+ * ---------------------------------------------------------------------------------------- */
+int cmx_mfma_tile_probe(const uint8_t* w, const uint8_t* ws, const uint8_t* a, const uint8_t* as, float* out,
+                        int fmt, cmx_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* CATCCOS_MX_H */

@@ -1,0 +1,84 @@
+"""The full single-device MoE FFN against the oracle chain."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import mx_oracle as O
+from catccos_amd import workloads as W
+from tests.gpu_util import dev, host, bf16_dev, close_bf16
+
+pytestmark = pytest.mark.gpu
+
+
+def _make(tokens, k, n, experts, top_k, seed):
+    rng = np.random.default_rng(seed)
+    x = W.normal_bf16((tokens, k), seed)
+    idx, p = W.softmax_topk_routing(tokens, experts, top_k, seed + 1)
+    w1 = [O.mx_quant(O.bf16_round(rng.standard_normal((n, k)).astype(np.float32) / np.sqrt(k)), "E4M3", "lut") for _ in range(experts)]
+    w2 = [O.mx_quant(O.bf16_round(rng.standard_normal((k, n // 2)).astype(np.float32) / np.sqrt(n // 2)), "E4M3", "lut") for _ in range(experts)]
+    w1q, w1s = np.stack([a for a, _ in w1]), np.stack([b for _, b in w1])
+    w2q, w2s = np.stack([a for a, _ in w2]), np.stack([b for _, b in w2])
+    return x, idx, p, w1q, w1s, w2q, w2s
+
+
+@pytest.mark.parametrize("tokens,k,n,experts,top_k", [(4, 256, 512, 4, 2), (64, 512, 1024, 16, 6), (300, 256, 512, 8, 8),
+                                                      (512, 512, 512, 32, 4)])
+def test_ffn_vs_oracle(tokens, k, n, experts, top_k):
+    from catccos_amd import ops
+    x, idx, p, w1q, w1s, w2q, w2s = _make(tokens, k, n, experts, top_k, seed=tokens)
+    ws_bytes = ops.ffn_workspace_bytes(tokens, k, n, experts, top_k)
+    workspace = torch.full((ws_bytes,), 0xA5, dtype=torch.uint8, device="cuda")      # poisoned, as the reference's regression mode
+    out = ops.dispatch_ffn_combine(bf16_dev(x), dev(idx), dev(p), dev(w1q), dev(w1s), dev(w2q), dev(w2s), workspace=workspace)
+    gold, st = O.moe_ffn(x, idx, p, w1q, w1s, w2q, w2s, stages=True)
+    got = host(out)
+    # End to end the chain holds two requantisations whose rounding decisions can flip on a
+    # one-ulp difference of the bf16 GMM1 output, so single elements may move by more than a
+    # matmul's tolerance: require 99.9% within rtol/atol 1e-2, none beyond 5e-2, and the
+    # reference's mean-bias bound; the matmul stages are checked one by one below.
+    gold_f = O.bf16_bits_to_f32(gold)
+    bad, worst = close_bf16(got, gold_f)
+    assert bad <= got.size // 1000 and worst <= 5e-2, (bad, worst)
+    ok, err, eb = O.verify_bf16(got, gold_f, 1 << 20)
+    assert eb <= 2.0 ** -7 and err <= got.size // 1000, (err, eb)
+    # integer stages are bit-exact: routing tables and the dispatched MX rows
+    lay = ops.ffn_workspace_layout(tokens, k, n, experts, top_k)
+    rows = tokens * top_k
+    w = workspace.cpu().numpy()
+    assert np.array_equal(w[lay["src2sorted"]:lay["src2sorted"] + rows * 4].view(np.int32), st["src2sorted"])
+    assert np.array_equal(w[lay["sorted2src"]:lay["sorted2src"] + rows * 4].view(np.int32), st["sorted2src"])
+    assert np.array_equal(w[lay["counts"]:lay["counts"] + experts * 4].view(np.int32), st["counts"])
+    assert np.array_equal(w[lay["a_codes"]:lay["a_codes"] + rows * k].reshape(rows, k), st["aq"])
+    assert np.array_equal(w[lay["a_scales"]:lay["a_scales"] + rows * (k // 32)].reshape(rows, k // 32), st["asc"])
+    # stage by stage on the kernel's own intermediates
+    half = n // 2
+    qa = w[lay["act_codes"]:lay["act_codes"] + rows * half].reshape(rows, half)
+    sa = w[lay["act_scales"]:lay["act_scales"] + rows * (half // 32)].reshape(rows, half // 32)
+    deq, deq_g = O.mx_dequant(qa, sa), O.mx_dequant(st["qa"], st["sa"])
+    bound = 0.13 * np.abs(deq_g) + 2.0 ** -5 * np.abs(deq_g).max(axis=1, keepdims=True)
+    assert np.all(np.abs(deq - deq_g) <= bound)
+    y = w[lay["y"]:lay["y"] + rows * k * 2].view(np.uint16).reshape(rows, k)
+    bad, worst = close_bf16(y, O.mx_gmm_f32(qa, sa, w2q, w2s, st["counts"]))          # GMM2 on the same codes
+    assert bad == 0, (bad, worst)
+    assert np.array_equal(got, O.unpermute_combine(y, st["src2sorted"], p))            # combine is bit-exact
+    # second launch on the same (now dirty) workspace gives the same bits
+    out2 = ops.dispatch_ffn_combine(bf16_dev(x), dev(idx), dev(p), dev(w1q), dev(w1s), dev(w2q), dev(w2s), workspace=workspace)
+    assert torch.equal(out, out2)
+
+
+def test_workspace_size_matches_reference_formula():
+    from catccos_amd import ops
+    for (m, k, n, e, t) in [(4, 7168, 4096, 16, 6), (512, 7168, 4096, 16, 6), (8192, 7168, 4096, 256, 8), (256, 7168, 1024, 16, 6)]:
+        assert ops.ffn_workspace_bytes(m, k, n, e, t) == O.ffn_workspace_bytes(m, k, n, 1, 1, e, t)
+        assert ops.ffn_workspace_layout(m, k, n, e, t)["y"] + m * t * k * 2 <= ops.ffn_workspace_bytes(m, k, n, e, t)
+
+
+def test_ffn_rejects_bad_shapes():
+    from catccos_amd import _lib
+    lib = _lib.load()
+    z = torch.zeros(1 << 20, dtype=torch.uint8, device="cuda")
+    p = z.data_ptr()
+    args = lambda m, k, n, e, t, r: (0, None, 0, p, p, p, p, p, p, p, p, p, None, m, k, n, e, t, r)
+    assert lib.catccos_ascend950_dispatch_ffn_combine(*args(4, 128, 512, 4, 2, 1)) == -1     # K % 256
+    assert lib.catccos_ascend950_dispatch_ffn_combine(*args(4, 256, 256, 4, 2, 1)) == -1     # N % 512
+    assert lib.catccos_ascend950_dispatch_ffn_combine(*args(4, 256, 512, 4, 5, 1)) == -1     # topK > experts
+    assert lib.catccos_ascend950_dispatch_ffn_combine(*args(4, 256, 512, 4, 2, 2)) == -1     # rankSize

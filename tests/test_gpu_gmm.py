@@ -1,0 +1,108 @@
+"""Grouped matmul over ragged expert groups, with and without the fused SwiGLU + requant."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import mx_oracle as O
+from catccos_amd import workloads as W
+from tests.gpu_util import dev, host, close_bf16
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(autouse=True)
+def _reset_tile():
+    yield
+    from catccos_amd import _lib
+    _lib.load().cmx_debug_force_tile(0, 0)
+
+
+def _weights(rng, g, n, k, std=0.05, fmt="E4M3"):
+    qs = [O.mx_quant(O.bf16_round(rng.standard_normal((n, k)).astype(np.float32) * std), fmt, "lut") for _ in range(g)]
+    return np.stack([q for q, _ in qs]), np.stack([s for _, s in qs])
+
+
+@pytest.mark.parametrize("tile", [None, (256, 256), (256, 128), (256, 64), (128, 128)])
+@pytest.mark.parametrize("counts", [[5, 0, 300, 1, 0, 257, 64], [0, 0, 7], [512], [1] * 9])
+def test_gmm_fp8_ragged_groups(tile, counts):
+    from catccos_amd import ops, _lib
+    if tile:
+        _lib.load().cmx_debug_force_tile(*tile)
+    rng = np.random.default_rng(sum(counts))
+    n, k = 320, 256
+    m = sum(counts)
+    aq, asc = O.mx_quant(O.bf16_round(rng.standard_normal((m + 3, k)).astype(np.float32)))
+    wq, ws = _weights(rng, len(counts), n, k, std=1.0)
+    c = torch.full((m + 3, n), 7.0, dtype=torch.bfloat16, device="cuda")
+    ops.mx_gmm(dev(aq), dev(asc), dev(wq), dev(ws), dev(np.array(counts, dtype=np.int32)), k, c=c)
+    got = host(c)
+    gold = O.mx_gmm_f32(aq[:m], asc[:m], wq, ws, counts)
+    bad, worst = close_bf16(got[:m], gold)
+    assert bad == 0, (bad, worst)
+    assert np.all(O.bf16_bits_to_f32(got[m:]) == 7.0)          # rows past the groups stay untouched
+
+
+def test_gmm_fp4_ragged_groups():
+    from catccos_amd import ops
+    rng = np.random.default_rng(3)
+    counts = [40, 0, 129, 300]
+    n, k = 256, 512
+    m = sum(counts)
+    aq, asc = O.mx_quant(rng.uniform(-2, 2, (m, k)).astype(np.float32), "E2M1")
+    ws_ = [O.mx_quant(rng.uniform(-2, 2, (n, k)).astype(np.float32), "E2M1") for _ in counts]
+    wq, ws = np.stack([q for q, _ in ws_]), np.stack([s for _, s in ws_])
+    c = ops.mx_gmm(dev(O.pack_fp4(aq)), dev(asc), dev(O.pack_fp4(wq)), dev(ws), dev(np.array(counts, dtype=np.int32)), k,
+                   "E2M1", "fp16")
+    gold = O.mx_gmm_f32(aq, asc, wq, ws, counts, "E2M1", "E2M1")
+    assert np.allclose(host(c).astype(np.float64), gold, rtol=2e-3, atol=5e-2)
+
+
+@pytest.mark.parametrize("tile", [None, (256, 256), (256, 128), (256, 64), (128, 128)])
+def test_gmm1_swiglu_requant(tile):
+    """h and act are within tolerance of the golden chain; the requantised codes and scales are
+    bit-exact against the oracle quantizer applied to the kernel's own bf16 SwiGLU output."""
+    from catccos_amd import ops, _lib
+    if tile:
+        _lib.load().cmx_debug_force_tile(*tile)
+    rng = np.random.default_rng(12)
+    counts = [70, 0, 300, 3, 130]
+    n, k = 512, 512
+    m = sum(counts)
+    aq, asc = O.mx_quant(O.bf16_round(rng.standard_normal((m, k)).astype(np.float32)))
+    wq, ws = _weights(rng, len(counts), n, k, std=0.06)
+    codes, scales, act = ops.mx_gmm_swiglu_quant(dev(aq), dev(asc), dev(wq), dev(ws),
+                                                 dev(np.array(counts, dtype=np.int32)), k, want_bf16=True)
+    h_g, act_g, q_g, s_g = O.gmm1_swiglu_quant(aq, asc, wq, ws, counts)
+    act_bits = host(act)
+    # gate and up are each rounded to bf16 before the product (+-2^-8 each) and the product is
+    # rounded again, so a one-ulp flip of either input moves act by up to ~1.2%: rtol 2e-2 here
+    bad, worst = close_bf16(act_bits, O.bf16_bits_to_f32(act_g), rtol=2e-2)
+    assert bad == 0, (bad, worst)
+    wq2, ws2 = O.mx_quant_bf16(act_bits, "E4M3", "rne")
+    assert np.array_equal(host(scales), ws2)
+    assert np.array_equal(host(codes), wq2)
+    # end to end the dequantised activations stay within tolerance of the golden's
+    deq = O.mx_dequant(host(codes), host(scales))
+    deq_g = O.mx_dequant(q_g, s_g)
+    # a flipped rounding decision moves an element by one E4M3 step (2^-3 relative), a flipped
+    # block exponent by one step of the coarser grid: bound by a step of the row's largest value
+    bound = 0.13 * np.abs(deq_g) + 2.0 ** -5 * np.abs(deq_g).max(axis=1, keepdims=True)
+    assert np.all(np.abs(deq - deq_g) <= bound)
+
+
+def test_config3_routing_shape_small_hidden():
+    """Zipf-routed ragged groups with two empty experts (the config-3 generator at reduced K/N)."""
+    from catccos_amd import ops
+    idx = W.zipf_routing(1024, 16, 8, seed=3)
+    counts = np.bincount(idx.reshape(-1), minlength=16).astype(np.int32)
+    assert (counts == 0).sum() == 2 and counts.sum() == 8192
+    rng = np.random.default_rng(4)
+    n, k = 512, 256
+    aq, asc = O.mx_quant(O.bf16_round(rng.standard_normal((8192, k)).astype(np.float32)))
+    wq, ws = _weights(rng, 16, n, k, std=0.08)
+    codes, scales, act = ops.mx_gmm_swiglu_quant(dev(aq), dev(asc), dev(wq), dev(ws), dev(counts), k, want_bf16=True)
+    _, act_g, _, _ = O.gmm1_swiglu_quant(aq, asc, wq, ws, counts)
+    bad, worst = close_bf16(host(act), O.bf16_bits_to_f32(act_g), rtol=2e-2)
+    assert bad == 0, (bad, worst)
+    wq2, ws2 = O.mx_quant_bf16(host(act), "E4M3", "rne")
+    assert np.array_equal(host(scales), ws2) and np.array_equal(host(codes), wq2)

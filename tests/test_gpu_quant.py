@@ -1,0 +1,125 @@
+"""Bit-exact parity of the HIP MX quantizer (through the C ABI) with the oracle."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import mx_oracle as O
+from catccos_amd import workloads as W
+from tests.gpu_util import dev, host, bf16_dev
+
+pytestmark = pytest.mark.gpu
+
+CASES = [("E4M3", "rne"), ("E4M3", "lut"), ("E5M2", "rne"), ("E5M2", "lut"), ("E2M1", "lut"), ("E2M1", "rne")]
+
+
+def _check(xbits, fmt, mode):
+    from catccos_amd import ops
+    q, s = ops.mx_quant(bf16_dev(xbits), fmt, mode)
+    wq, ws = O.mx_quant_bf16(xbits, fmt, mode)
+    if fmt == "E2M1":
+        wq = O.pack_fp4(wq)
+    gq, gs = host(q), host(s)
+    assert np.array_equal(gs, ws), f"scales differ at {np.argwhere(gs != ws)[:5]}"
+    assert np.array_equal(gq, wq), f"codes differ: {np.count_nonzero(gq != wq)} of {gq.size}"
+
+
+@pytest.mark.parametrize("fmt,mode", CASES)
+def test_every_bf16_value_in_varied_company(fmt, mode):
+    """All 65536 bf16 patterns (finite ones), each placed in blocks whose amax is set by a
+    different neighbour so every value meets many shared exponents, ties and clips included."""
+    bits = np.arange(65536, dtype=np.uint16)
+    fin = np.isfinite(O.bf16_bits_to_f32(bits))
+    bits = bits[fin]
+    rng = np.random.default_rng(11)
+    rows = []
+    for shift in (0, 3, 7, 64, 200):
+        b = np.roll(bits, shift * 131)
+        pad = (-b.size) % 32
+        b = np.concatenate([b, np.zeros(pad, dtype=np.uint16)])
+        blocks = b.reshape(-1, 32).copy()
+        if shift:
+            blocks = blocks[rng.permutation(blocks.shape[0])]
+            blocks = rng.permuted(blocks, axis=1)
+        rows.append(blocks.reshape(-1, 256))
+    _check(np.concatenate(rows, axis=0), fmt, mode)
+
+
+@pytest.mark.parametrize("fmt,mode", CASES)
+def test_exact_midpoints_and_clips(fmt, mode):
+    """Every midpoint between adjacent grid values (where RNE and table rounding part ways) and
+    values between the largest grid value and 2x it (clip), in blocks whose scale is 2^0."""
+    tab = {"E4M3": O.e4m3_table()[:127], "E5M2": O.e5m2_table()[:124], "E2M1": O.fp4_table()[:8]}[fmt]
+    top = float(tab[-1])
+    mids = ((tab[:-1].astype(np.float64) + tab[1:]) / 2).astype(np.float32)
+    mids = mids[O.bf16_round(mids) == mids]          # those exactly representable in bf16
+    emax = O.FORMATS[fmt]["emax"]
+    anchor = np.float32(2.0 ** emax)                 # amax with floor(log2) = emax -> shared exponent 0
+    vals = np.concatenate([mids, -mids, tab, -tab, np.linspace(top, 2 * top * 0.99, 40).astype(np.float32)])
+    vals = vals[np.abs(vals) < 2 * anchor]
+    x = np.zeros((vals.size, 32), dtype=np.float32)
+    x[:, 0] = anchor
+    x[:, 1] = vals
+    xb = O.f32_to_bf16_bits(x)
+    q, s = O.mx_quant_bf16(xb, fmt, mode)
+    keep = s[:, 0] == 127
+    assert keep.sum() > vals.size // 2
+    _check(xb.reshape(-1, 32), fmt, mode)
+
+
+@pytest.mark.parametrize("rows,cols", [(1, 32), (3, 40), (5, 20), (7, 96), (2, 7168), (33, 1000), (4, 2050)])
+def test_ragged_shapes(rows, cols):
+    xb = W.activations_with_outliers(rows, cols, seed=rows * 1000 + cols)
+    for fmt, mode in [("E4M3", "rne"), ("E2M1", "lut")]:
+        _check(xb, fmt, mode)
+
+
+def test_zero_and_tiny_blocks():
+    x = np.zeros((4, 64), dtype=np.float32)
+    x[1, :32] = 1e-13          # below epsilon: scale stays 2^0, elements flush to zero codes
+    x[2, 0] = -0.0
+    x[3, 5] = 2.0 ** -120
+    _check(O.f32_to_bf16_bits(x), "E4M3", "rne")
+    _check(O.f32_to_bf16_bits(x), "E4M3", "lut")
+    _check(O.f32_to_bf16_bits(x), "E2M1", "lut")
+
+
+def test_row_pitches():
+    from catccos_amd import _lib
+    xb = W.activations_with_outliers(16, 256, seed=5)
+    big = torch.zeros((16, 512), dtype=torch.int16, device="cuda")
+    big[:, :256] = dev(xb)
+    codes = torch.full((16, 320), 0xAA, dtype=torch.uint8, device="cuda")
+    scales = torch.full((16, 16), 0xBB, dtype=torch.uint8, device="cuda")
+    lib = _lib.load()
+    _lib.check(lib.cmx_mx_quant(big.data_ptr(), 512, codes.data_ptr(), 320, scales.data_ptr(), 16, 16, 256, 0, 0,
+                                torch.cuda.current_stream().cuda_stream))
+    wq, ws = O.mx_quant_bf16(xb)
+    assert np.array_equal(host(codes)[:, :256], wq) and np.all(host(codes)[:, 256:] == 0xAA)
+    assert np.array_equal(host(scales)[:, :8], ws) and np.all(host(scales)[:, 8:] == 0xBB)
+
+
+def test_config1_shape_bit_exact_and_idempotent():
+    """bf16 [4096, 7168], N(0,1) with 0.1% outliers x100: bit-exact vs the oracle, then the
+    reference's byte-exact protocol: re-quantising the dequantised output reproduces it."""
+    from catccos_amd import ops
+    xb = W.activations_with_outliers(4096, 7168, seed=1)
+    q, s = ops.mx_quant(bf16_dev(xb), "E4M3", "rne")
+    wq, ws = O.mx_quant_bf16(xb)
+    assert np.array_equal(host(s), ws) and np.array_equal(host(q), wq)
+    deq = ops.mx_dequant(q, s, 7168)
+    assert np.array_equal(host(deq), O.mx_dequant(wq, ws))
+    q2, s2 = ops.mx_quant(deq.to(torch.bfloat16), "E4M3", "rne")
+    assert torch.equal(q2, q) and torch.equal(s2, s)
+
+
+def test_bad_arguments_are_rejected():
+    from catccos_amd import _lib
+    lib = _lib.load()
+    x = torch.zeros((4, 64), dtype=torch.int16, device="cuda")
+    c = torch.zeros((4, 64), dtype=torch.uint8, device="cuda")
+    s = torch.zeros((4, 2), dtype=torch.uint8, device="cuda")
+    assert lib.cmx_mx_quant(x.data_ptr(), 64, c.data_ptr(), 64, s.data_ptr(), 2, 4, 64, 9, 0, None) == -1
+    assert lib.cmx_mx_quant(x.data_ptr(), 32, c.data_ptr(), 64, s.data_ptr(), 2, 4, 64, 0, 0, None) == -1
+    assert lib.cmx_mx_quant(None, 64, c.data_ptr(), 64, s.data_ptr(), 2, 4, 64, 0, 0, None) == -1
+    assert b"pitch" in lib.cmx_last_error() or b"null" in lib.cmx_last_error()
+    assert lib.cmx_mx_quant(x.data_ptr(), 64, c.data_ptr(), 64, s.data_ptr(), 2, 0, 64, 0, 0, None) == 0   # empty
