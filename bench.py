@@ -1,0 +1,277 @@
+#!/usr/bin/env python3
+"""Benchmark of the MI355X MX compute core (one GPU).
+
+Headline step = one pass of the MoE grouped matmul with fused dequant + SwiGLU + MX requant
+(BASELINE.json config 3: E=16 local experts, 4096 tokens x top-8 Zipf-routed = 32768 ragged rows,
+H=7168, W_gate/up [16, 4096, 7168] MXFP8) through the C ABI, inputs resident in HBM.
+`value` = 2*rows*K*N flop / step time in TFLOP/s.  The same JSON line carries
+
+  roofline      the grouped-matmul kernel against the dense MXFP8 MFMA peak (HIP-event timing on the
+                launch stream), and in `extra` the quantizer / dense GEMM / FFN / FP4 / routing kernels
+                each against its own bound;
+  cpu_baseline  the numpy oracle of the same step timed on the host cores over a bounded sample.
+
+Usage: python bench.py [--gpus 1] [--steps K] [--warmup W] [--only NAME[,NAME]] [--no-cpu]
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0
+MXFP8_PEAK_TFLOPS = 5000.0
+MXFP4_PEAK_TFLOPS = 10100.0
+SEED = 20240607
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--only", type=str, default="", help="comma list of extras: quant,gemm,ffn,fp4,routing (default all)")
+    ap.add_argument("--no-extras", action="store_true")
+    ap.add_argument("--no-cpu", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build measures one GPU's share of the path; --gpus must be 1 "
+              "(no collectives, no multi-device sharding in this tier)", file=sys.stderr)
+        return 2
+
+    import torch
+    from catccos_amd import _lib, ops, workloads as W
+
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        return 3
+    lib = _lib.load()          # raises if the HIP library is missing: there is no fallback
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    K_STEPS, WARM = args.steps, args.warmup
+
+    def hip_time(fn, steps=K_STEPS, warm=WARM):
+        """Average duration (s) of fn() over `steps` launches, HIP events on the launch stream."""
+        for _ in range(warm):
+            fn()
+        torch.cuda.synchronize()
+        e0 = torch.cuda.Event(enable_timing=True)
+        e1 = torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(steps):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) * 1e-3 / steps
+
+    def quant_weights(e, n, k, std, seed):
+        """[e, n, k] MXFP8 weights: N(0, std) bf16 quantised per expert by the GPU quantizer (table rounding)."""
+        g = torch.Generator(device=dev)
+        g.manual_seed(seed)
+        codes = torch.empty((e, n, k), dtype=torch.uint8, device=dev)
+        scales = torch.empty((e, n, ops.scale_cols(k)), dtype=torch.uint8, device=dev)
+        for i in range(e):
+            w = (torch.randn((n, k), generator=g, device=dev) * std).to(torch.bfloat16)
+            q, s = ops.mx_quant(w, "E4M3", "lut")
+            codes[i], scales[i] = q, s
+        return codes, scales
+
+    # ------------------------------------------------------------------ headline: config 3 ----
+    E, T, TOPK, H, N = 16, 4096, 8, 7168, 4096
+    idx = W.zipf_routing(T, E, TOPK, SEED)
+    counts_h = np.bincount(idx.reshape(-1), minlength=E).astype(np.int32)
+    rows = int(counts_h.sum())
+    counts = torch.from_numpy(counts_h).to(dev)
+    g = torch.Generator(device=dev)
+    g.manual_seed(SEED)
+    xa = torch.randn((rows, H), generator=g, device=dev).to(torch.bfloat16)
+    a_codes, a_scales = ops.mx_quant(xa, "E4M3", "rne")
+    del xa
+    w1, w1s = quant_weights(E, N, H, 0.02, SEED + 1)
+    act_codes = torch.empty((rows, N // 2), dtype=torch.uint8, device=dev)
+    act_scales = torch.empty((rows, ops.scale_cols(N // 2)), dtype=torch.uint8, device=dev)
+    gws = ops.gmm_workspace(E, dev)
+
+    def step():
+        ops.mx_gmm_swiglu_quant(a_codes, a_scales, w1, w1s, counts, H, workspace=gws, outs=(act_codes, act_scales))
+
+    for _ in range(WARM):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(K_STEPS):
+        step()
+    torch.cuda.synchronize()
+    wall = (time.perf_counter() - t0) / K_STEPS
+    flop = 2.0 * rows * H * N
+    value = flop / wall / 1e12
+    kern = hip_time(step)
+    log(f"[gmm1+swiglu+requant cfg3] wall {wall*1e6:.1f} us/step, events {kern*1e6:.1f} us -> {flop/kern/1e12:.0f} TFLOP/s")
+    roofline = {"kernel": "mx_gemm_kernel<E4M3, swiglu+requant epilogue> (grouped, config 3)", "bound": "mfma",
+                "achieved": flop / kern / 1e12, "peak": MXFP8_PEAK_TFLOPS, "unit": "TFLOP/s",
+                "frac": flop / kern / 1e12 / MXFP8_PEAK_TFLOPS, "traffic": None,
+                "flop_per_launch": flop, "avg_launch_us": kern * 1e6}
+
+    # ------------------------------------------------------------------ CPU baseline -----------
+    cpu = None
+    if not args.no_cpu:
+        from oracle import mx_oracle as O
+        sample_groups = [i for i in np.argsort(-counts_h)[:2]]
+        cap = 1024
+        off = np.concatenate([[0], np.cumsum(counts_h)])
+        a_h, as_h = [], []
+        cnt = []
+        for gi in sample_groups:
+            r = min(cap, int(counts_h[gi]))
+            a_h.append(a_codes[off[gi]:off[gi] + r].cpu().numpy())
+            as_h.append(a_scales[off[gi]:off[gi] + r].cpu().numpy())
+            cnt.append(r)
+        a_h, as_h = np.concatenate(a_h), np.concatenate(as_h)
+        w_h = w1[sample_groups].cpu().numpy()
+        ws_h = w1s[sample_groups].cpu().numpy()
+        O.gmm1_swiglu_quant(a_h[:64], as_h[:64], w_h, ws_h, [32, 32])        # warm-up
+        reps = []
+        for _ in range(3):
+            t0 = time.perf_counter()
+            O.gmm1_swiglu_quant(a_h, as_h, w_h, ws_h, cnt)
+            reps.append(time.perf_counter() - t0)
+        tc = float(np.median(reps))
+        cflop = 2.0 * sum(cnt) * H * N
+        cores = len(os.sched_getaffinity(0))
+        omp = os.environ.get("OMP_NUM_THREADS")
+        if omp and omp.isdigit():
+            cores = min(cores, int(omp))
+        cpu = {"value": cflop / tc / 1e12, "unit": "TFLOP/s", "cores": cores, "kind": "port",
+               "sample": f"numpy oracle gmm1_swiglu_quant on {len(cnt)} experts x {cnt} rows (K={H}, N={N}), "
+                         f"median of 3 = {tc:.2f} s; includes dequantising operands to fp32"}
+        log(f"[cpu baseline] {cpu['value']*1e3:.1f} GFLOP/s on {cores} threads ({tc:.2f} s)")
+        del a_h, as_h, w_h, ws_h
+
+    # ------------------------------------------------------------------ extras -----------------
+    extra = {}
+    want = set(x for x in args.only.split(",") if x) or {"quant", "gemm", "ffn", "fp4", "routing"}
+    if args.no_extras:
+        want = set()
+
+    if "quant" in want:
+        M1, K1 = 4096, 7168
+        x1 = torch.from_numpy(W.activations_with_outliers(M1, K1, SEED).view(np.int16)).to(dev)
+        q1 = torch.empty((M1, K1), dtype=torch.uint8, device=dev)
+        s1 = torch.empty((M1, K1 // 32), dtype=torch.uint8, device=dev)
+        st = torch.cuda.current_stream().cuda_stream
+        tq = hip_time(lambda: lib.cmx_mx_quant(x1.data_ptr(), K1, q1.data_ptr(), K1, s1.data_ptr(), K1 // 32, M1, K1, 0, 0, st),
+                      steps=max(K_STEPS, 50))
+        bytes_q = M1 * K1 * 2 + M1 * K1 + M1 * K1 // 32
+        extra["mx_quant_cfg1"] = {"kernel": "mx_quant_kernel<E4M3, RNE>", "bound": "hbm", "achieved": bytes_q / tq / 1e9,
+                                  "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": bytes_q / tq / 1e9 / HBM_PEAK_GBS,
+                                  "bytes_per_launch": bytes_q, "avg_launch_us": tq * 1e6, "traffic": None}
+        log(f"[mx_quant cfg1] {tq*1e6:.1f} us -> {bytes_q/tq/1e9:.0f} GB/s")
+        del x1, q1, s1
+
+    if "gemm" in want:
+        M2, N2, K2 = 8192, 4096, 7168
+        g.manual_seed(SEED + 2)
+        a2, a2s = ops.mx_quant(torch.randn((M2, K2), generator=g, device=dev).to(torch.bfloat16))
+        b2, b2s = ops.mx_quant(torch.randn((N2, K2), generator=g, device=dev).to(torch.bfloat16))
+        tg = hip_time(lambda: ops.mx_gemm(a2, a2s, b2, b2s, K2))
+        fl2 = 2.0 * M2 * N2 * K2
+        extra["mx_gemm_cfg2"] = {"kernel": "mx_gemm_kernel<E4M3, store epilogue> (dense)", "bound": "mfma",
+                                 "achieved": fl2 / tg / 1e12, "peak": MXFP8_PEAK_TFLOPS, "unit": "TFLOP/s",
+                                 "frac": fl2 / tg / 1e12 / MXFP8_PEAK_TFLOPS, "avg_launch_us": tg * 1e6}
+        log(f"[mx_gemm cfg2] {tg*1e6:.1f} us -> {fl2/tg/1e12:.0f} TFLOP/s")
+        del a2, a2s, b2, b2s
+
+    if "fp4" in want:
+        E5, T5, K5, N5 = 32, 8192, 7168, 4096
+        idx5 = W.zipf_routing(T5, E5, 8, SEED + 5)
+        c5h = np.bincount(idx5.reshape(-1), minlength=E5).astype(np.int32)
+        rows5 = int(c5h.sum())
+        c5 = torch.from_numpy(c5h).to(dev)
+        g.manual_seed(SEED + 5)
+        a5, a5s = ops.mx_quant((torch.rand((rows5, K5), generator=g, device=dev) * 4 - 2).to(torch.bfloat16), "E2M1", "lut")
+        w5 = torch.empty((E5, N5, K5 // 2), dtype=torch.uint8, device=dev)
+        w5s = torch.empty((E5, N5, K5 // 32), dtype=torch.uint8, device=dev)
+        for i in range(E5):
+            q, s = ops.mx_quant((torch.rand((N5, K5), generator=g, device=dev) * 4 - 2).to(torch.bfloat16), "E2M1", "lut")
+            w5[i], w5s[i] = q, s
+        c_out = torch.empty((rows5, N5), dtype=torch.bfloat16, device=dev)
+        ws5 = ops.gmm_workspace(E5, dev)
+        t5 = hip_time(lambda: ops.mx_gmm(a5, a5s, w5, w5s, c5, K5, "E2M1", "bf16", c=c_out, workspace=ws5))
+        fl5 = 2.0 * rows5 * K5 * N5
+        extra["mxfp4_gmm_cfg5"] = {"kernel": "mx_gemm_kernel<E2M1, store epilogue> (grouped)", "bound": "mfma",
+                                   "achieved": fl5 / t5 / 1e12, "peak": MXFP4_PEAK_TFLOPS, "unit": "TFLOP/s",
+                                   "frac": fl5 / t5 / 1e12 / MXFP4_PEAK_TFLOPS, "avg_launch_us": t5 * 1e6}
+        log(f"[mxfp4 gmm cfg5] {t5*1e6:.1f} us -> {fl5/t5/1e12:.0f} TFLOP/s")
+        del a5, a5s, w5, w5s, c_out
+
+    if "ffn" in want or "routing" in want:
+        T4, E4, K4, N4, TOP4 = 8192, 256, 7168, 4096, 8
+        idx4, p4 = W.softmax_topk_routing(T4, E4, TOP4, SEED + 4)
+        idx4_d, p4_d = torch.from_numpy(idx4).to(dev), torch.from_numpy(p4).to(dev)
+        g.manual_seed(SEED + 4)
+        x4 = torch.randn((T4, K4), generator=g, device=dev).to(torch.bfloat16)
+        rows4 = T4 * TOP4
+        if "routing" in want:
+            s2s, inv, cnt4 = ops.moe_init_routing(idx4_d, E4)
+            ts = hip_time(lambda: ops.moe_init_routing(idx4_d, E4))
+            qa = torch.empty((rows4, K4), dtype=torch.uint8, device=dev)
+            qs = torch.empty((rows4, K4 // 32), dtype=torch.uint8, device=dev)
+            st = torch.cuda.current_stream().cuda_stream
+            tqs = hip_time(lambda: lib.cmx_quant_scatter(x4.data_ptr(), K4, inv.data_ptr(), qa.data_ptr(), K4, qs.data_ptr(),
+                                                         K4 // 32, T4, K4, TOP4, st))
+            b_qs = T4 * K4 * 2 + rows4 * (K4 + K4 // 32)
+            y4 = torch.randn((rows4, K4), generator=g, device=dev).to(torch.bfloat16)
+            tc4 = hip_time(lambda: ops.moe_token_unpermute(y4, inv, p4_d))
+            b_c = rows4 * K4 * 2 + T4 * K4 * 2
+            extra["routing_cfg4"] = {
+                "expert_sort_us": ts * 1e6,
+                "quant_scatter": {"bound": "hbm", "achieved": b_qs / tqs / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                                  "frac": b_qs / tqs / 1e9 / HBM_PEAK_GBS, "avg_launch_us": tqs * 1e6},
+                "unpermute_combine": {"bound": "hbm", "achieved": b_c / tc4 / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                                      "frac": b_c / tc4 / 1e9 / HBM_PEAK_GBS, "avg_launch_us": tc4 * 1e6}}
+            log(f"[routing cfg4] sort {ts*1e6:.1f} us, quant_scatter {b_qs/tqs/1e9:.0f} GB/s, combine {b_c/tc4/1e9:.0f} GB/s")
+            del qa, qs, y4
+        if "ffn" in want:
+            w14, w14s = quant_weights(E4, N4, K4, 0.02, SEED + 6)
+            w24, w24s = quant_weights(E4, K4, N4 // 2, 0.02, SEED + 7)
+            wsp = torch.empty(ops.ffn_workspace_bytes(T4, K4, N4, E4, TOP4), dtype=torch.uint8, device=dev)
+            out4 = torch.empty((T4, K4), dtype=torch.bfloat16, device=dev)
+            tf = hip_time(lambda: ops.dispatch_ffn_combine(x4, idx4_d, p4_d, w14, w14s, w24, w24s, workspace=wsp, out=out4),
+                          steps=max(5, K_STEPS // 2), warm=2)
+            fl4 = 2.0 * rows4 * K4 * (N4 + N4 // 2)
+            by4 = float(w14.numel() + w14s.numel() + w24.numel() + w24s.numel()) + T4 * K4 * 2 \
+                + 2 * rows4 * (K4 + K4 // 32) + 2 * rows4 * (N4 // 2 + N4 // 64) + 2 * rows4 * K4 * 2 + T4 * K4 * 2
+            extra["moe_ffn_cfg4"] = {"ms": tf * 1e3, "tflops": fl4 / tf / 1e12, "mfma_frac": fl4 / tf / 1e12 / MXFP8_PEAK_TFLOPS,
+                                     "algorithmic_GB": by4 / 1e9, "hbm_GBs": by4 / tf / 1e9, "hbm_frac": by4 / tf / 1e9 / HBM_PEAK_GBS,
+                                     "tokens_per_s": T4 / tf}
+            log(f"[moe ffn cfg4] {tf*1e3:.3f} ms -> {fl4/tf/1e12:.0f} TFLOP/s, {by4/tf/1e9:.0f} GB/s algorithmic")
+
+    line = {
+        "metric": "MXFP8 GMM TFLOP/s (% MFMA peak); MX-quant GB/s (% HBM peak), 1 GPU",
+        "value": value, "unit": "TFLOP/s", "n_gpus": 1, "steps": K_STEPS, "warmup": WARM,
+        "ms_per_step": wall * 1e3, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "mxfp8 (E4M3 elements, E8M0 block-32 scales), fp32 accumulate", "data": "synthetic",
+        "config": {"workload": "config 3: MoE grouped matmul + dequant + SwiGLU + MX requant, E=16, 4096 tokens x top-8 "
+                               "Zipf(1.1) routed (2 empty experts), H=7168, W [16,4096,7168] MXFP8",
+                   "rows": rows, "K": H, "N": N, "experts": E, "seed": SEED,
+                   "group_sizes": counts_h.tolist()},
+        "mfma_peak_frac": value / MXFP8_PEAK_TFLOPS,
+        "roofline": roofline, "cpu_baseline": cpu, "extra": extra,
+    }
+    print(json.dumps(line), flush=True)
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())
