@@ -9,7 +9,8 @@ import ctypes as C
 import os
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "lib", "libcatccos_mx.so")
+# CATCCOS_MX_LIB points at another build of the same library (e.g. an experimental kernel variant)
+LIB_PATH = os.environ.get("CATCCOS_MX_LIB") or os.path.join(_HERE, "lib", "libcatccos_mx.so")
 
 u8p, i32p, f32p, vp = C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p
 u32, i32, u64, sz = C.c_uint32, C.c_int, C.c_uint64, C.c_size_t
@@ -55,7 +56,8 @@ SIGNATURES = {
                                                      u32, u32, u32, u32, u32, i32]),
     "cmx_ffn_workspace_layout_get": (i32, [u32, u32, u32, u32, u32, C.POINTER(FfnWorkspaceLayout)]),
     "cmx_mfma_raw_probe": (i32, [vp, vp, i32p, i32p, f32p, i32, i32, i32, vp]),
-    "cmx_debug_force_tile": (i32, [i32, i32]),
+    "cmx_debug_force_tile": (i32, [i32, i32, i32]),
+    "cmx_debug_disable_streaming": (i32, [i32]),
 }
 
 _lib = None

@@ -20,13 +20,14 @@
 // that prefix, so no host synchronisation is needed and empty groups cost nothing.  Workgroup ids
 // are remapped so that each XCD (ids congruent mod 8) walks a contiguous run of tiles that share
 // weight panels in its own L2.
+#include <type_traits>
+
 #include "mx_common.h"
 
 namespace cmx {
 
 namespace {
 
-constexpr int kThreads = 256;
 constexpr int kSlabBytes = 128;     // K bytes per LDS slab and row
 constexpr int kChunks = kSlabBytes / 16;
 constexpr int kXcds = 8;
@@ -100,245 +101,67 @@ __device__ __forceinline__ float silu_mul(float g, float u) {
     return (g * s) * u;
 }
 
-// TW/TM: tile rows (weights / activations); WW x WM wavefront grid over the tile.
-template <int FMT, int TW, int TM, int WW, int WM, int EPI>
-__global__ __launch_bounds__(kThreads) void mx_gemm_kernel(const GemmParams p) {
-    static_assert(WW * WM == 4, "four wavefronts per workgroup");
-    constexpr bool kFp4 = FMT == CMX_FMT_E2M1;
-    constexpr int kSub = kFp4 ? 4 : 2;                 // MFMA steps (64 K elements each) per slab
-    constexpr int kScaleDw = kFp4 ? 2 : 1;             // scale dwords per row per slab
-    constexpr int FW = TW / WW / 32;                   // 32-row fragments per wavefront, weights
-    constexpr int FM = TM / WM / 32;                   // activations
-    constexpr int kWLoads = TW / 32;                   // 16-byte chunks per thread per slab
-    constexpr int kALoads = TM / 32;
-    static_assert(EPI == kEpiStore || (FW % 2 == 0), "gate/up fragments come in pairs");
-    constexpr int kStageBytes = (TW + TM) * kSlabBytes + (TW + TM) * 4 * kScaleDw;
+struct Tile {
+    uint32_t g, mt, wt, row0, rows_valid;
+};
 
-    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
-
-    const uint32_t tid = threadIdx.x;
-    const uint32_t lane = tid & 63u;
-    const uint32_t wave = tid >> 6;
-    const uint32_t ww = wave % WW, wm = wave / WW;
-
-    // ---- which tile -------------------------------------------------------------------------
-    uint32_t total_tiles, g = 0, mt, wt, row0, rows_valid;
-    {
-        const uint32_t grouped = p.row_off != nullptr;
-        uint32_t m_tiles_all = grouped ? (uint32_t)p.tile_pref[p.groups] : (p.m + TM - 1) / TM;
-        total_tiles = m_tiles_all * p.w_tiles;
-        const uint32_t bid = blockIdx.x;
-        if (bid >= total_tiles) return;
-        // XCD-aware remap: ids congruent mod 8 run on one XCD; give each a contiguous run.
-        const uint32_t x = bid % kXcds, j = bid / kXcds;
-        const uint32_t base = total_tiles / kXcds, rem = total_tiles % kXcds;
-        const uint32_t L = x * base + (x < rem ? x : rem) + j;
-        if (grouped) {
-            // find g with tile_pref[g]*w_tiles <= L < tile_pref[g+1]*w_tiles
-            uint32_t lo = 0, hi = p.groups;
-            while (hi - lo > 1) {
-                uint32_t mid = (lo + hi) >> 1;
-                if ((uint32_t)p.tile_pref[mid] * p.w_tiles <= L) lo = mid; else hi = mid;
-            }
-            g = lo;
-            const uint32_t tp = (uint32_t)p.tile_pref[g];
-            const uint32_t mtg = (uint32_t)p.tile_pref[g + 1] - tp;
-            const uint32_t local = L - tp * p.w_tiles;
-            mt = local % mtg;
-            wt = local / mtg;
-            const uint32_t r_begin = (uint32_t)p.row_off[g], r_end = (uint32_t)p.row_off[g + 1];
-            row0 = r_begin + mt * TM;
-            rows_valid = r_end - row0 < (uint32_t)TM ? r_end - row0 : (uint32_t)TM;
-        } else {
-            // groups of 4 m-tiles share a run of weight tiles
-            const uint32_t m_tiles = m_tiles_all;
-            const uint32_t band = 4;
-            const uint32_t per_band = band * p.w_tiles;
-            const uint32_t b = L / per_band, within = L % per_band;
-            const uint32_t band_rows = (m_tiles - b * band) < band ? (m_tiles - b * band) : band;
-            mt = b * band + within % band_rows;
-            wt = within / band_rows;
-            row0 = mt * TM;
-            rows_valid = p.m - row0 < (uint32_t)TM ? p.m - row0 : (uint32_t)TM;
+// Maps the workgroup id to (group, m-tile, weight tile).  Returns false for ids past the last tile.
+template <int TM>
+__device__ __forceinline__ bool locate_tile(const GemmParams& p, Tile& t) {
+    const uint32_t grouped = p.row_off != nullptr;
+    const uint32_t m_tiles_all = grouped ? (uint32_t)p.tile_pref[p.groups] : (p.m + TM - 1) / TM;
+    const uint32_t total_tiles = m_tiles_all * p.w_tiles;
+    const uint32_t bid = blockIdx.x;
+    if (bid >= total_tiles) return false;
+    // XCD-aware remap: ids congruent mod 8 run on one XCD; give each a contiguous run of tiles.
+    const uint32_t x = bid % kXcds, j = bid / kXcds;
+    const uint32_t base = total_tiles / kXcds, rem = total_tiles % kXcds;
+    const uint32_t L = x * base + (x < rem ? x : rem) + j;
+    if (grouped) {
+        // find g with tile_pref[g]*w_tiles <= L < tile_pref[g+1]*w_tiles
+        uint32_t lo = 0, hi = p.groups;
+        while (hi - lo > 1) {
+            const uint32_t mid = (lo + hi) >> 1;
+            if ((uint32_t)p.tile_pref[mid] * p.w_tiles <= L) lo = mid; else hi = mid;
         }
+        t.g = lo;
+        const uint32_t tp = (uint32_t)p.tile_pref[lo];
+        const uint32_t mtg = (uint32_t)p.tile_pref[lo + 1] - tp;
+        const uint32_t local = L - tp * p.w_tiles;
+        t.mt = local % mtg;             // m fastest: neighbours share the weight panel
+        t.wt = local / mtg;
+        const uint32_t r_begin = (uint32_t)p.row_off[lo], r_end = (uint32_t)p.row_off[lo + 1];
+        t.row0 = r_begin + t.mt * TM;
+        t.rows_valid = r_end - t.row0 < (uint32_t)TM ? r_end - t.row0 : (uint32_t)TM;
+    } else {
+        // bands of 4 m-tiles share a run of weight tiles
+        const uint32_t band = 4;
+        const uint32_t per_band = band * p.w_tiles;
+        const uint32_t b = L / per_band, within = L % per_band;
+        const uint32_t band_rows = (m_tiles_all - b * band) < band ? (m_tiles_all - b * band) : band;
+        t.g = 0;
+        t.mt = b * band + within % band_rows;
+        t.wt = within / band_rows;
+        t.row0 = t.mt * TM;
+        t.rows_valid = p.m - t.row0 < (uint32_t)TM ? p.m - t.row0 : (uint32_t)TM;
     }
+    return true;
+}
 
-    // ---- global -> LDS staging assignments -----------------------------------------------------
-    const uint32_t ld_chunk = tid & 7u;        // 16-byte chunk inside the slab
-    const uint32_t ld_row = tid >> 3;          // + 32*j
-    const uint8_t* wg = p.w + (size_t)g * p.n * p.ldw;
-    const uint8_t* wsg = p.w_scale + (size_t)g * p.n * p.ld_ws;
+// LDS/tile row of a wavefront's weight fragment f (gate fragments first, their up partners second)
+template <int TW, int WW, int EPI, int FW>
+__device__ __forceinline__ uint32_t wfrag_row_of(uint32_t ww, int f) {
+    if (EPI == kEpiSwigluQuant)
+        return f < FW / 2 ? ww * (TW / 2 / WW) + f * 32 : TW / 2 + ww * (TW / 2 / WW) + (f - FW / 2) * 32;
+    return ww * (TW / WW) + f * 32;
+}
 
-    // global weight row of LDS tile row r
-    auto wrow_of = [&](uint32_t r) -> uint32_t {
-        uint32_t gr;
-        if (EPI == kEpiSwigluQuant) {
-            const uint32_t half = p.n >> 1;
-            uint32_t rr = r < TW / 2 ? wt * (TW / 2) + r : wt * (TW / 2) + (r - TW / 2);
-            rr = rr < half ? rr : half - 1;
-            gr = r < TW / 2 ? rr : half + rr;
-        } else {
-            gr = wt * TW + r;
-            gr = gr < p.n ? gr : p.n - 1;
-        }
-        return gr;
-    };
-    auto arow_of = [&](uint32_t r) -> uint32_t { return row0 + (r < rows_valid ? r : rows_valid - 1); };
-
-    const uint8_t* wptr[kWLoads];
-    const uint8_t* aptr[kALoads];
-#pragma unroll
-    for (int j = 0; j < kWLoads; ++j) wptr[j] = wg + (size_t)wrow_of(ld_row + 32 * j) * p.ldw + ld_chunk * 16;
-#pragma unroll
-    for (int j = 0; j < kALoads; ++j) aptr[j] = p.a + (size_t)arow_of(ld_row + 32 * j) * p.lda + ld_chunk * 16;
-    // scale rows: thread t serves weight row t (t < TW) and activation row t (t < TM)
-    const uint8_t* wsptr = wsg + (size_t)wrow_of(tid < TW ? tid : 0) * p.ld_ws;
-    const uint8_t* asptr = p.a_scale + (size_t)arow_of(tid < TM ? tid : 0) * p.ld_as;
-
-    const uint32_t nslab = (p.kbytes + kSlabBytes - 1) / kSlabBytes;
-    const uint32_t blocks_per_slab = 4 * kScaleDw;
-
-    uint4 wreg[kWLoads], areg[kALoads];
-    uint32_t wsreg[kScaleDw], asreg[kScaleDw];
-
-    auto load_scale_dw = [&](const uint8_t* rowp, uint32_t blk0) -> uint32_t {
-        // four consecutive scale bytes starting at block blk0; beyond K the scale is 1.0
-        if (p.scale_vec && blk0 + 4 <= p.kblocks) return *reinterpret_cast<const uint32_t*>(rowp + blk0);
-        uint32_t v = 0x7F7F7F7Fu;
-        for (uint32_t i = 0; i < 4; ++i)
-            if (blk0 + i < p.kblocks) v = (v & ~(0xFFu << (8 * i))) | ((uint32_t)rowp[blk0 + i] << (8 * i));
-        return v;
-    };
-    auto load_global = [&](uint32_t slab) {
-        const uint32_t kb = slab * kSlabBytes + ld_chunk * 16;
-        const bool in = kb < p.kbytes;
-#pragma unroll
-        for (int j = 0; j < kWLoads; ++j)
-            wreg[j] = in ? *reinterpret_cast<const uint4*>(wptr[j] + (size_t)slab * kSlabBytes) : make_uint4(0, 0, 0, 0);
-#pragma unroll
-        for (int j = 0; j < kALoads; ++j)
-            areg[j] = in ? *reinterpret_cast<const uint4*>(aptr[j] + (size_t)slab * kSlabBytes) : make_uint4(0, 0, 0, 0);
-#pragma unroll
-        for (int d = 0; d < kScaleDw; ++d) {
-            const uint32_t blk0 = slab * blocks_per_slab + 4 * d;
-            if (tid < TW) wsreg[d] = load_scale_dw(wsptr, blk0);
-            if (tid < TM) asreg[d] = load_scale_dw(asptr, blk0);
-        }
-    };
-    auto store_lds = [&](uint32_t stage) {
-        uint8_t* sW = smem + stage * kStageBytes;
-        uint8_t* sA = sW + TW * kSlabBytes;
-        uint32_t* sWs = reinterpret_cast<uint32_t*>(sA + TM * kSlabBytes);
-        uint32_t* sAs = sWs + TW * kScaleDw;
-#pragma unroll
-        for (int j = 0; j < kWLoads; ++j) {
-            const uint32_t r = ld_row + 32 * j;
-            *reinterpret_cast<uint4*>(sW + r * kSlabBytes + swz(r, ld_chunk) * 16) = wreg[j];
-        }
-#pragma unroll
-        for (int j = 0; j < kALoads; ++j) {
-            const uint32_t r = ld_row + 32 * j;
-            *reinterpret_cast<uint4*>(sA + r * kSlabBytes + swz(r, ld_chunk) * 16) = areg[j];
-        }
-#pragma unroll
-        for (int d = 0; d < kScaleDw; ++d) {
-            if (tid < TW) sWs[tid * kScaleDw + d] = wsreg[d];
-            if (tid < TM) sAs[tid * kScaleDw + d] = asreg[d];
-        }
-    };
-
-    // ---- accumulators --------------------------------------------------------------------------
-    v16f acc[FW][FM];
-#pragma unroll
-    for (int i = 0; i < FW; ++i)
-#pragma unroll
-        for (int j = 0; j < FM; ++j)
-#pragma unroll
-            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
-
-    // LDS row of the wavefront's fragment f
-    auto wfrag_row = [&](int f) -> uint32_t {
-        if (EPI == kEpiSwigluQuant)
-            return f < FW / 2 ? ww * (TW / 2 / WW) + f * 32 : TW / 2 + ww * (TW / 2 / WW) + (f - FW / 2) * 32;
-        return ww * (TW / WW) + f * 32;
-    };
+template <int TW, int TM, int WW, int WM, int EPI, int FW, int FM>
+__device__ __forceinline__ void epilogue(const GemmParams& p, const Tile& tc, v16f (&acc)[FW][FM], uint32_t ww,
+                                         uint32_t wm, uint32_t lane) {
     const uint32_t l32 = lane & 31u, lh = lane >> 5;
-
-    auto compute = [&](uint32_t stage) {
-        const uint8_t* sW = smem + stage * kStageBytes;
-        const uint8_t* sA = sW + TW * kSlabBytes;
-        const uint32_t* sWs = reinterpret_cast<const uint32_t*>(sA + TM * kSlabBytes);
-        const uint32_t* sAs = sWs + TW * kScaleDw;
-        // lane's scale registers: byte 2*h' (after the lh shift) belongs to MFMA step h' of the dword
-        uint32_t sw[FW][kScaleDw], sa[FM][kScaleDw];
-#pragma unroll
-        for (int f = 0; f < FW; ++f)
-#pragma unroll
-            for (int d = 0; d < kScaleDw; ++d) sw[f][d] = sWs[(wfrag_row(f) + l32) * kScaleDw + d] >> (8 * lh);
-#pragma unroll
-        for (int f = 0; f < FM; ++f)
-#pragma unroll
-            for (int d = 0; d < kScaleDw; ++d)
-                sa[f][d] = sAs[(wm * (TM / WM) + f * 32 + l32) * kScaleDw + d] >> (8 * lh);
-
-#pragma unroll
-        for (int h = 0; h < kSub; ++h) {
-            v8i af[FM];
-#pragma unroll
-            for (int f = 0; f < FM; ++f) {
-                const uint32_t r = wm * (TM / WM) + f * 32 + l32;
-                const uint8_t* rp = sA + r * kSlabBytes;
-                if (kFp4) {
-                    const uint32_t c0 = h * 2 + lh;
-                    v4i lo = *reinterpret_cast<const v4i*>(rp + swz(r, c0) * 16);
-                    af[f] = (v8i){lo[0], lo[1], lo[2], lo[3], 0, 0, 0, 0};
-                } else {
-                    // 8-bit operands: registers 0-3 carry k = 16*lh + [0,16) of the step's first
-                    // 32-block, registers 4-7 the same slice of its second 32-block
-                    const uint32_t c0 = h * 4 + lh;
-                    v4i lo = *reinterpret_cast<const v4i*>(rp + swz(r, c0) * 16);
-                    v4i hi = *reinterpret_cast<const v4i*>(rp + swz(r, c0 + 2) * 16);
-                    af[f] = (v8i){lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-                }
-            }
-#pragma unroll
-            for (int fw = 0; fw < FW; ++fw) {
-                const uint32_t r = wfrag_row(fw) + l32;
-                const uint8_t* rp = sW + r * kSlabBytes;
-                v8i wf;
-                if (kFp4) {
-                    const uint32_t c0 = h * 2 + lh;
-                    v4i lo = *reinterpret_cast<const v4i*>(rp + swz(r, c0) * 16);
-                    wf = (v8i){lo[0], lo[1], lo[2], lo[3], 0, 0, 0, 0};
-                } else {
-                    const uint32_t c0 = h * 4 + lh;
-                    v4i lo = *reinterpret_cast<const v4i*>(rp + swz(r, c0) * 16);
-                    v4i hi = *reinterpret_cast<const v4i*>(rp + swz(r, c0 + 2) * 16);
-                    wf = (v8i){lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-                }
-#pragma unroll
-                for (int fm = 0; fm < FM; ++fm) {
-                    // step h uses scale dword h/2, byte 2*(h%2) of the shifted register
-                    acc[fw][fm] = mfma<FMT>(wf, af[fm], acc[fw][fm], (h & 1) * 2, (int)sw[fw][h >> 1],
-                                            (int)sa[fm][h >> 1]);
-                }
-            }
-        }
-    };
-
-    // ---- main loop -------------------------------------------------------------------------------
-    load_global(0);
-    store_lds(0);
-    __syncthreads();
-    for (uint32_t s = 0; s < nslab; ++s) {
-        const bool more = s + 1 < nslab;
-        if (more) load_global(s + 1);
-        compute(s & 1u);
-        if (more) store_lds((s + 1) & 1u);
-        __syncthreads();
-    }
-
-    // ---- epilogue ----------------------------------------------------------------------------------
+    const uint32_t wt = tc.wt, row0 = tc.row0, rows_valid = tc.rows_valid;
+    auto wfrag_row = [&](int f) -> uint32_t { return wfrag_row_of<TW, WW, EPI, FW>(ww, f); };
     if constexpr (EPI == kEpiStore) {
 #pragma unroll
         for (int fm = 0; fm < FM; ++fm) {
@@ -425,6 +248,467 @@ __global__ __launch_bounds__(kThreads) void mx_gemm_kernel(const GemmParams p) {
     }
 }
 
+// TW/TM: tile rows (weights / activations); WW x WM wavefront grid over the tile (4 or 8 wavefronts).
+// FAST: K is a whole number of slabs and scale rows are dword aligned, so the main loop carries no
+// bounds checks at all.
+template <int FMT, int TW, int TM, int WW, int WM, int EPI, bool FAST>
+__global__ __launch_bounds__(64 * WW * WM) void mx_gemm_kernel(const GemmParams p) {
+    constexpr int NT = 64 * WW * WM;
+    static_assert(NT == 256 || NT == 512, "four or eight wavefronts per workgroup");
+    constexpr bool kFp4 = FMT == CMX_FMT_E2M1;
+    constexpr int kSub = kFp4 ? 4 : 2;                 // MFMA steps (64 K elements each) per slab
+    constexpr int kScaleDw = kFp4 ? 2 : 1;             // scale dwords per row per slab
+    constexpr int FW = TW / WW / 32;                   // 32-row fragments per wavefront, weights
+    constexpr int FM = TM / WM / 32;                   // activations
+    constexpr int kRowsPerPass = NT / kChunks;         // tile rows covered by one 16-byte load per thread
+    constexpr int kWLoads = TW / kRowsPerPass;         // 16-byte chunks per thread per slab
+    constexpr int kALoads = TM / kRowsPerPass;
+    static_assert(FW >= 1 && FM >= 1 && kWLoads >= 1 && kALoads >= 1, "tile too small for the wavefront grid");
+    static_assert(EPI == kEpiStore || (FW % 2 == 0), "gate/up fragments come in pairs");
+    static_assert(TW <= NT && TM <= NT, "one scale row per thread");
+    constexpr int kStageBytes = (TW + TM) * kSlabBytes + (TW + TM) * 4 * kScaleDw;
+
+    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+
+    const uint32_t tid = threadIdx.x;
+    const uint32_t lane = tid & 63u;
+    const uint32_t wave = tid >> 6;
+    const uint32_t ww = wave % WW, wm = wave / WW;
+
+    Tile tc;
+    if (!locate_tile<TM>(p, tc)) return;
+    const uint32_t g = tc.g, wt = tc.wt, row0 = tc.row0, rows_valid = tc.rows_valid;
+
+    // ---- global -> LDS staging assignments -----------------------------------------------------
+    const uint32_t ld_chunk = tid & 7u;                // 16-byte chunk inside the slab
+    const uint32_t ld_row = tid >> 3;                  // + kRowsPerPass*j
+    const uint8_t* wg = p.w + (size_t)g * p.n * p.ldw;             // uniform bases, 32-bit lane offsets
+    const uint8_t* wsg = p.w_scale + (size_t)g * p.n * p.ld_ws;
+    const uint8_t* ag = p.a + (size_t)row0 * p.lda;
+    const uint8_t* asg = p.a_scale + (size_t)row0 * p.ld_as;
+
+    // global weight row of LDS tile row r (rows past the matrix repeat the last one; masked at the store)
+    auto wrow_of = [&](uint32_t r) -> uint32_t {
+        uint32_t gr;
+        if (EPI == kEpiSwigluQuant) {
+            const uint32_t half = p.n >> 1;
+            uint32_t rr = r < TW / 2 ? wt * (TW / 2) + r : wt * (TW / 2) + (r - TW / 2);
+            rr = rr < half ? rr : half - 1;
+            gr = r < TW / 2 ? rr : half + rr;
+        } else {
+            gr = wt * TW + r;
+            gr = gr < p.n ? gr : p.n - 1;
+        }
+        return gr;
+    };
+    auto arow_of = [&](uint32_t r) -> uint32_t { return r < rows_valid ? r : rows_valid - 1; };
+
+    uint32_t woff[kWLoads], aoff[kALoads];
+#pragma unroll
+    for (int j = 0; j < kWLoads; ++j) woff[j] = wrow_of(ld_row + kRowsPerPass * j) * p.ldw + ld_chunk * 16;
+#pragma unroll
+    for (int j = 0; j < kALoads; ++j) aoff[j] = arow_of(ld_row + kRowsPerPass * j) * p.lda + ld_chunk * 16;
+    // scale rows: thread t serves weight row t (t < TW) and activation row t (t < TM)
+    const uint32_t wsoff = wrow_of(tid < TW ? tid : 0) * p.ld_ws;
+    const uint32_t asoff = arow_of(tid < TM ? tid : 0) * p.ld_as;
+
+    const uint32_t nslab = (p.kbytes + kSlabBytes - 1) / kSlabBytes;
+    constexpr uint32_t blocks_per_slab = 4 * kScaleDw;
+
+    uint4 wreg[kWLoads], areg[kALoads];
+    uint32_t wsreg[kScaleDw], asreg[kScaleDw];
+
+    auto load_scale_dw = [&](const uint8_t* rowp, uint32_t blk0) -> uint32_t {
+        // four consecutive scale bytes starting at block blk0; beyond K the scale is 1.0
+        if (FAST || (p.scale_vec && blk0 + 4 <= p.kblocks)) return *reinterpret_cast<const uint32_t*>(rowp + blk0);
+        uint32_t v = 0x7F7F7F7Fu;
+        for (uint32_t i = 0; i < 4; ++i)
+            if (blk0 + i < p.kblocks) v = (v & ~(0xFFu << (8 * i))) | ((uint32_t)rowp[blk0 + i] << (8 * i));
+        return v;
+    };
+    auto load_global = [&](uint32_t slab) {
+        const uint8_t* wslab = wg + (size_t)slab * kSlabBytes;
+        const uint8_t* aslab = ag + (size_t)slab * kSlabBytes;
+        const bool in = FAST || (slab * kSlabBytes + ld_chunk * 16 < p.kbytes);
+#pragma unroll
+        for (int j = 0; j < kWLoads; ++j)
+            wreg[j] = in ? *reinterpret_cast<const uint4*>(wslab + woff[j]) : make_uint4(0, 0, 0, 0);
+#pragma unroll
+        for (int j = 0; j < kALoads; ++j)
+            areg[j] = in ? *reinterpret_cast<const uint4*>(aslab + aoff[j]) : make_uint4(0, 0, 0, 0);
+#pragma unroll
+        for (int d = 0; d < kScaleDw; ++d) {
+            const uint32_t blk0 = slab * blocks_per_slab + 4 * d;
+            if (tid < TW) wsreg[d] = load_scale_dw(wsg + wsoff, blk0);
+            if (tid < TM) asreg[d] = load_scale_dw(asg + asoff, blk0);
+        }
+    };
+    auto store_lds = [&](uint32_t stage) {
+        uint8_t* sW = smem + stage * kStageBytes;
+        uint8_t* sA = sW + TW * kSlabBytes;
+        uint32_t* sWs = reinterpret_cast<uint32_t*>(sA + TM * kSlabBytes);
+        uint32_t* sAs = sWs + TW * kScaleDw;
+#pragma unroll
+        for (int j = 0; j < kWLoads; ++j) {
+            const uint32_t r = ld_row + kRowsPerPass * j;
+            *reinterpret_cast<uint4*>(sW + r * kSlabBytes + swz(r, ld_chunk) * 16) = wreg[j];
+        }
+#pragma unroll
+        for (int j = 0; j < kALoads; ++j) {
+            const uint32_t r = ld_row + kRowsPerPass * j;
+            *reinterpret_cast<uint4*>(sA + r * kSlabBytes + swz(r, ld_chunk) * 16) = areg[j];
+        }
+#pragma unroll
+        for (int d = 0; d < kScaleDw; ++d) {
+            if (tid < TW) sWs[tid * kScaleDw + d] = wsreg[d];
+            if (tid < TM) sAs[tid * kScaleDw + d] = asreg[d];
+        }
+    };
+
+    // ---- accumulators --------------------------------------------------------------------------
+    v16f acc[FW][FM];
+#pragma unroll
+    for (int i = 0; i < FW; ++i)
+#pragma unroll
+        for (int j = 0; j < FM; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+
+    auto wfrag_row = [&](int f) -> uint32_t { return wfrag_row_of<TW, WW, EPI, FW>(ww, f); };
+    const uint32_t l32 = lane & 31u, lh = lane >> 5;
+
+    // byte offsets (within a stage's W / A tile) of the lane's two 16-byte runs for step 0; the runs
+    // of step h sit at chunk index + 4h (8-bit) or + 2h (FP4), i.e. the XOR swizzle is re-applied
+    auto frag_addr = [&](uint32_t r, uint32_t c) -> uint32_t { return r * kSlabBytes + swz(r, c) * 16; };
+
+    auto read_frag = [&](const uint8_t* tile, uint32_t r, int h) -> v8i {
+        if (kFp4) {
+            v4i lo = *reinterpret_cast<const v4i*>(tile + frag_addr(r, h * 2 + lh));
+            return (v8i){lo[0], lo[1], lo[2], lo[3], 0, 0, 0, 0};
+        }
+        // 8-bit operands: registers 0-3 carry k = 16*lh + [0,16) of the step's first 32-block,
+        // registers 4-7 the same slice of its second 32-block
+        v4i lo = *reinterpret_cast<const v4i*>(tile + frag_addr(r, h * 4 + lh));
+        v4i hi = *reinterpret_cast<const v4i*>(tile + frag_addr(r, h * 4 + lh + 2));
+        return (v8i){lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+    };
+
+    auto compute = [&](uint32_t stage) {
+        const uint8_t* sW = smem + stage * kStageBytes;
+        const uint8_t* sA = sW + TW * kSlabBytes;
+        const uint32_t* sWs = reinterpret_cast<const uint32_t*>(sA + TM * kSlabBytes);
+        const uint32_t* sAs = sWs + TW * kScaleDw;
+        // operand fragments are double buffered in registers: the LDS reads of step h+1 are issued
+        // before the MFMAs of step h
+        v8i af[2][FM], wf[2][FW];
+#pragma unroll
+        for (int f = 0; f < FM; ++f) af[0][f] = read_frag(sA, wm * (TM / WM) + f * 32 + l32, 0);
+#pragma unroll
+        for (int f = 0; f < FW; ++f) wf[0][f] = read_frag(sW, wfrag_row(f) + l32, 0);
+        // lane's scale registers: byte 2*h' (after the lh shift) belongs to MFMA step h' of the dword
+        uint32_t sw[FW][kScaleDw], sa[FM][kScaleDw];
+#pragma unroll
+        for (int f = 0; f < FW; ++f)
+#pragma unroll
+            for (int d = 0; d < kScaleDw; ++d) sw[f][d] = sWs[(wfrag_row(f) + l32) * kScaleDw + d] >> (8 * lh);
+#pragma unroll
+        for (int f = 0; f < FM; ++f)
+#pragma unroll
+            for (int d = 0; d < kScaleDw; ++d)
+                sa[f][d] = sAs[(wm * (TM / WM) + f * 32 + l32) * kScaleDw + d] >> (8 * lh);
+
+#pragma unroll
+        for (int h = 0; h < kSub; ++h) {
+            const int cur = h & 1, nxt = cur ^ 1;
+            if (h + 1 < kSub) {
+#pragma unroll
+                for (int f = 0; f < FM; ++f) af[nxt][f] = read_frag(sA, wm * (TM / WM) + f * 32 + l32, h + 1);
+#pragma unroll
+                for (int f = 0; f < FW; ++f) wf[nxt][f] = read_frag(sW, wfrag_row(f) + l32, h + 1);
+            }
+#pragma unroll
+            for (int fw = 0; fw < FW; ++fw) {
+#pragma unroll
+                for (int fm = 0; fm < FM; ++fm) {
+                    // step h uses scale dword h/2, byte 2*(h%2) of the shifted register
+                    acc[fw][fm] = mfma<FMT>(wf[cur][fw], af[cur][fm], acc[fw][fm], (h & 1) * 2, (int)sw[fw][h >> 1],
+                                            (int)sa[fm][h >> 1]);
+                }
+            }
+        }
+    };
+
+    // ---- main loop -------------------------------------------------------------------------------
+    load_global(0);
+    store_lds(0);
+    __syncthreads();
+    // steady state is branch free: prefetch slab s+1, consume slab s, refill the other stage
+    for (uint32_t s = 0; s + 1 < nslab; ++s) {
+#if !(defined(CMX_DBG_SKIP) && (CMX_DBG_SKIP & 1))
+        load_global(s + 1);
+#endif
+        __builtin_amdgcn_sched_barrier(0);
+#if !(defined(CMX_DBG_SKIP) && (CMX_DBG_SKIP & 2))
+        compute(s & 1u);
+#endif
+        // Keep the LDS refill (which waits for the global loads) behind the MFMAs of this slab: without
+        // a use of the accumulators here the compiler sinks the MFMAs below the refill and the barrier,
+        // which exposes the whole global-load latency every iteration.
+#pragma unroll
+        for (int i = 0; i < FW; ++i)
+#pragma unroll
+            for (int j = 0; j < FM; ++j) asm volatile("" ::"a"(acc[i][j][0]) : "memory");
+        __builtin_amdgcn_sched_barrier(0);
+#if !(defined(CMX_DBG_SKIP) && (CMX_DBG_SKIP & 4))
+        store_lds((s + 1) & 1u);
+#endif
+        __syncthreads();
+    }
+    compute((nslab - 1) & 1u);
+
+    epilogue<TW, TM, WW, WM, EPI, FW, FM>(p, tc, acc, ww, wm, lane);
+}
+
+// ------------------------------------------------------------------------------------------------
+// Streaming kernel: operand tiles go global -> LDS directly (LDS-DMA loads, no staging registers and
+// no ds_write) into a two-slot ring of 128-byte-deep K slabs; whole 128-byte lines per row keep every
+// fetched cache line fully used.  Operand fragments are prefetched into a spare register set one MFMA
+// step ahead, so a slot is drained one step before its slab's MFMAs end; at that point
+//   wait (own reads of slot s and own loads of slab s+1 done) -> barrier (everyone's) ->
+//   refill slot s with slab s+2 -> read the first fragments of slab s+1 -> last MFMA step of slab s.
+// One barrier per slab; every load has a full slab of MFMA time to land.
+// A load instruction of one wavefront fills 1 KiB of LDS linearly (lane p -> 16 bytes at 16p), i.e.
+// 8 tile rows x 8 chunks; the XOR swizzle that keeps the row-strided fragment reads conflict-free is
+// applied on the global side (which 16 bytes of the row a lane fetches).  Scale dwords (4 blocks each)
+// ride in their own two-slot ring.
+#define CMX_WAIT_VMCNT(n) __builtin_amdgcn_s_waitcnt(((n) & 0xF) | (((n) >> 4) << 14) | 0x0F70)
+#define CMX_WAIT_ALL() __builtin_amdgcn_s_waitcnt(0x0070)   // vmcnt(0) lgkmcnt(0)
+
+typedef __attribute__((address_space(3))) void* lds_void_ptr;
+typedef const __attribute__((address_space(1))) void* global_void_ptr;
+
+template <int FMT, int TW, int TM, int WW, int WM, int EPI>
+__global__ __launch_bounds__(64 * WW * WM) void mx_gemm_dl_kernel(const GemmParams p) {
+    constexpr int NW = WW * WM;                        // wavefronts: 4 (one per SIMD) or 8 (two per SIMD)
+    static_assert(NW == 4 || NW == 8, "four or eight wavefronts per workgroup");
+    constexpr bool kFp4 = FMT == CMX_FMT_E2M1;
+    constexpr int kSub = kFp4 ? 4 : 2;                 // MFMA steps (64 K elements each) per slab
+    constexpr int kScaleDw = kFp4 ? 2 : 1;             // scale dwords per row per slab
+    constexpr int FW = TW / WW / 32, FM = TM / WM / 32;
+    constexpr int kRows = TW + TM;                     // W tile rows then A tile rows
+    constexpr int kTileLoads = kRows / (8 * NW);       // direct loads per thread and slab (8 rows per wavefront-load)
+    constexpr int kWTileLoads = TW / (8 * NW);
+    constexpr int kSlotBytes = kRows * kSlabBytes;
+    constexpr int kScaleSlot = kRows * kScaleDw;       // dwords
+    constexpr int kScaleWaveLoads = kRows / 64;        // wavefront-loads that cover one scale dword of every row
+    constexpr int kScalePerWave = (kScaleWaveLoads + NW - 1) / NW;
+    constexpr int kLoadsPerSlab = kTileLoads + kScalePerWave * kScaleDw;
+    static_assert(TW % (8 * NW) == 0 && TM % (8 * NW) == 0 && TW % 64 == 0 && TM % 64 == 0, "tile shape");
+    static_assert(FW >= 1 && FM >= 1, "tile too small for the wavefront grid");
+    static_assert(EPI == kEpiStore || (FW % 2 == 0), "gate/up fragments come in pairs");
+
+    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+    uint32_t* const sScale = reinterpret_cast<uint32_t*>(smem + 2 * kSlotBytes);
+
+    const uint32_t tid = threadIdx.x;
+    const uint32_t lane = tid & 63u;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const uint32_t ww = wave % WW, wm = wave / WW;
+    const uint32_t l32 = lane & 31u, lh = lane >> 5;
+
+    Tile tc;
+    if (!locate_tile<TM>(p, tc)) return;
+    const uint32_t g = __builtin_amdgcn_readfirstlane(tc.g), wt = __builtin_amdgcn_readfirstlane(tc.wt);
+    const uint32_t row0 = __builtin_amdgcn_readfirstlane(tc.row0);
+    const uint32_t rows_valid = __builtin_amdgcn_readfirstlane(tc.rows_valid);
+
+    const uint8_t* wg = p.w + (size_t)g * p.n * p.ldw;
+    const uint8_t* wsg = p.w_scale + (size_t)g * p.n * p.ld_ws;
+    const uint8_t* ag = p.a + (size_t)row0 * p.lda;
+    const uint8_t* asg = p.a_scale + (size_t)row0 * p.ld_as;
+
+    auto wrow_of = [&](uint32_t r) -> uint32_t {
+        uint32_t gr;
+        if (EPI == kEpiSwigluQuant) {
+            const uint32_t half = p.n >> 1;
+            uint32_t rr = r < TW / 2 ? wt * (TW / 2) + r : wt * (TW / 2) + (r - TW / 2);
+            rr = rr < half ? rr : half - 1;
+            gr = r < TW / 2 ? rr : half + rr;
+        } else {
+            gr = wt * TW + r;
+            gr = gr < p.n ? gr : p.n - 1;
+        }
+        return gr;
+    };
+    auto arow_of = [&](uint32_t r) -> uint32_t { return r < rows_valid ? r : rows_valid - 1; };
+
+    // ---- per-lane offsets of the direct loads --------------------------------------------------
+    // load i of this wavefront fills combined tile rows (NW*i + wave)*8 .. +8; lane p -> row +p/8, LDS chunk p%8
+    uint32_t goff[kTileLoads];
+#pragma unroll
+    for (int i = 0; i < kTileLoads; ++i) {
+        const uint32_t cr = (NW * i + wave) * 8 + (lane >> 3);
+        const uint32_t logical = swz(cr, lane & 7u);
+        goff[i] = (i < kWTileLoads ? wrow_of(cr) * p.ldw : arow_of(cr - TW) * p.lda) + logical * 16;
+    }
+    // scale dwords: one wavefront-load covers 64 rows; wavefront-load j serves W rows 64j.. (j < TW/64) or A rows
+    uint32_t soff_[kScalePerWave], sdst_[kScalePerWave];
+    bool s_is_w[kScalePerWave];
+#pragma unroll
+    for (int t = 0; t < kScalePerWave; ++t) {
+        const uint32_t j = wave + NW * t;
+        s_is_w[t] = j < TW / 64;
+        const uint32_t aj = (j - TW / 64) % (TM / 64);
+        soff_[t] = s_is_w[t] ? wrow_of(64 * j + lane) * p.ld_ws : arow_of(64 * aj + lane) * p.ld_as;
+        sdst_[t] = s_is_w[t] ? 64 * j : TW + 64 * aj;
+    }
+
+    const uint32_t nslab = p.kbytes / kSlabBytes;
+
+    // Buffer addressing: per-lane byte offsets stay constant over the whole K loop and the slab
+    // position is a scalar offset, so a load costs no vector ALU work at all.
+    constexpr int kRsrcFlags = 0x00020000;
+    auto uniform_ptr = [](const uint8_t* q) -> uint8_t* {
+        const uint64_t v = reinterpret_cast<uint64_t>(q);
+        const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v), hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
+        return reinterpret_cast<uint8_t*>(((uint64_t)hi << 32) | lo);
+    };
+    const __amdgpu_buffer_rsrc_t w_rs = __builtin_amdgcn_make_buffer_rsrc(uniform_ptr(wg), 0, -1, kRsrcFlags);
+    const __amdgpu_buffer_rsrc_t a_rs = __builtin_amdgcn_make_buffer_rsrc(uniform_ptr(ag), 0, -1, kRsrcFlags);
+    const __amdgpu_buffer_rsrc_t ws_rs = __builtin_amdgcn_make_buffer_rsrc(uniform_ptr(wsg), 0, -1, kRsrcFlags);
+    const __amdgpu_buffer_rsrc_t as_rs = __builtin_amdgcn_make_buffer_rsrc(uniform_ptr(asg), 0, -1, kRsrcFlags);
+
+    auto issue_slab = [&](uint32_t slab) {
+        const uint32_t k = slab < nslab ? slab : nslab - 1;              // past the end: harmless reload
+        uint8_t* dst = smem + (slab & 1u) * kSlotBytes + wave * 1024;
+        const int koff = (int)(k * kSlabBytes);
+#pragma unroll
+        for (int i = 0; i < kTileLoads; ++i) {
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(i < kWTileLoads ? w_rs : a_rs, (lds_void_ptr)(dst + i * (NW * 1024)), 16,
+                                                     (int)goff[i], koff, 0, 0);
+        }
+        uint32_t* sdst = sScale + (slab & 1u) * kScaleSlot;
+#pragma unroll
+        for (int d = 0; d < kScaleDw; ++d) {
+            const int soff = (int)((k * kScaleDw + d) * 4);
+#pragma unroll
+            for (int t = 0; t < kScalePerWave; ++t) {
+                if (s_is_w[t])
+                    __builtin_amdgcn_raw_ptr_buffer_load_lds(ws_rs, (lds_void_ptr)(sdst + d * kRows + sdst_[t]), 4, (int)soff_[t], soff, 0, 0);
+                else
+                    __builtin_amdgcn_raw_ptr_buffer_load_lds(as_rs, (lds_void_ptr)(sdst + d * kRows + sdst_[t]), 4, (int)soff_[t], soff, 0, 0);
+            }
+        }
+    };
+
+    // ---- fragment reads ------------------------------------------------------------------------
+    auto wfrag_row = [&](int f) -> uint32_t { return wfrag_row_of<TW, WW, EPI, FW>(ww, f); };
+    auto read_frag = [&](const uint8_t* tile, uint32_t r, int h) -> v8i {
+        const uint8_t* rp = tile + r * kSlabBytes;
+        if (kFp4) {
+            v4i lo = *reinterpret_cast<const v4i*>(rp + swz(r, h * 2 + lh) * 16);
+            return (v8i){lo[0], lo[1], lo[2], lo[3], 0, 0, 0, 0};
+        }
+        // 8-bit operands: registers 0-3 carry k = 16*lh + [0,16) of the step's first 32-block,
+        // registers 4-7 the same slice of its second 32-block
+        v4i lo = *reinterpret_cast<const v4i*>(rp + swz(r, h * 4 + lh) * 16);
+        v4i hi = *reinterpret_cast<const v4i*>(rp + swz(r, h * 4 + lh + 2) * 16);
+        return (v8i){lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+    };
+
+    v16f acc[FW][FM];
+#pragma unroll
+    for (int i = 0; i < FW; ++i)
+#pragma unroll
+        for (int j = 0; j < FM; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+
+    v8i wf[2][FW], af[2][FM];
+    uint32_t sw[kScaleDw][FW], sa[kScaleDw][FM], swn[kScaleDw][FW], san[kScaleDw][FM];
+
+    auto read_frags = [&](uint32_t slab, int h, int buf) {
+        const uint8_t* st = smem + (slab & 1u) * kSlotBytes;
+#pragma unroll
+        for (int f = 0; f < FM; ++f) af[buf][f] = read_frag(st + TW * kSlabBytes, wm * (TM / WM) + f * 32 + l32, h);
+#pragma unroll
+        for (int f = 0; f < FW; ++f) wf[buf][f] = read_frag(st, wfrag_row(f) + l32, h);
+    };
+    auto read_scales = [&](uint32_t slab, uint32_t (&w_)[kScaleDw][FW], uint32_t (&a_)[kScaleDw][FM]) {
+        const uint32_t* sc = sScale + (slab & 1u) * kScaleSlot;
+#pragma unroll
+        for (int d = 0; d < kScaleDw; ++d) {
+#pragma unroll
+            for (int f = 0; f < FW; ++f) w_[d][f] = sc[d * kRows + wfrag_row(f) + l32] >> (8 * lh);
+#pragma unroll
+            for (int f = 0; f < FM; ++f) a_[d][f] = sc[d * kRows + TW + wm * (TM / WM) + f * 32 + l32] >> (8 * lh);
+        }
+    };
+
+    // ---- prologue -----------------------------------------------------------------------------------
+    issue_slab(0);
+    issue_slab(1);
+    CMX_WAIT_VMCNT(kLoadsPerSlab);      // slab 0 has landed (slab 1 may still be in flight)
+    __syncthreads();
+    read_frags(0, 0, 0);
+    read_scales(0, sw, sa);
+
+    for (uint32_t s = 0; s < nslab; ++s) {
+#pragma unroll
+        for (int h = 0; h < kSub; ++h) {
+#ifndef CMX_DBG_SKIP
+#define CMX_DBG_SKIP 0
+#endif
+            if (h + 1 < kSub) {
+                if (!(CMX_DBG_SKIP & 8)) read_frags(s, h + 1, (h + 1) & 1);
+            } else {
+                // slot s&1 is drained by this wavefront one step early: refill point
+                if (!(CMX_DBG_SKIP & 16)) {
+                CMX_WAIT_ALL();                 // own fragment reads of slab s and own loads of slab s+1 are done
+                __syncthreads();                // ... and everyone else's
+                }
+                if (!(CMX_DBG_SKIP & 1)) issue_slab(s + 2);
+                if (!(CMX_DBG_SKIP & 8)) read_frags(s + 1, 0, 0);
+                if (!(CMX_DBG_SKIP & 8)) read_scales(s + 1, swn, san);
+            }
+            // One wavefront per SIMD issues in order, so the MFMA pipe idles whenever more than one
+            // MFMA time of other instructions sits between two MFMAs: spread the LDS reads and the
+            // LDS-DMA loads of this step evenly behind the MFMAs instead of clustering them.
+            {
+                constexpr int kMfmas = FW * FM;
+                constexpr int kFragReads = (FW + FM) * (kFp4 ? 1 : 2);
+                constexpr int kDs = kFragReads + (FW + FM) * kScaleDw;     // refill step also reads the scales
+                constexpr int kDsPer = (kDs + kMfmas - 1) / kMfmas;
+                constexpr int kVmPer = (kLoadsPerSlab + kMfmas - 1) / kMfmas;
+#pragma unroll
+                for (int i = 0; i < kMfmas; ++i) {
+                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);          // one MFMA
+                    if (h + 1 == kSub) __builtin_amdgcn_sched_group_barrier(0x020, kVmPer, 0);   // VMEM reads
+                    __builtin_amdgcn_sched_group_barrier(0x100, kDsPer, 0);     // DS reads
+                }
+            }
+#pragma unroll
+            for (int fw = 0; fw < FW; ++fw)
+#pragma unroll
+                for (int fm = 0; fm < FM; ++fm)
+                    acc[fw][fm] = mfma<FMT>(wf[h & 1][fw], af[h & 1][fm], acc[fw][fm], (h & 1) * 2, (int)sw[h >> 1][fw],
+                                            (int)sa[h >> 1][fm]);
+            // ... and this step's MFMAs must be issued before the next step's wait/barrier
+            __builtin_amdgcn_sched_barrier(0);
+        }
+#pragma unroll
+        for (int d = 0; d < kScaleDw; ++d) {
+#pragma unroll
+            for (int f = 0; f < FW; ++f) sw[d][f] = swn[d][f];
+#pragma unroll
+            for (int f = 0; f < FM; ++f) sa[d][f] = san[d][f];
+        }
+    }
+    CMX_WAIT_VMCNT(0);      // the two reloads issued past the end must land before the LDS is released
+
+    epilogue<TW, TM, WW, WM, EPI, FW, FM>(p, tc, acc, ww, wm, lane);
+}
+
 // Row offsets and m-tile prefix of the groups (one workgroup).
 __global__ void gmm_prepare_kernel(const int32_t* __restrict__ sizes, uint32_t groups, uint32_t tile_m,
                                    int32_t* __restrict__ row_off, int32_t* __restrict__ tile_pref) {
@@ -444,11 +728,11 @@ __global__ void gmm_prepare_kernel(const int32_t* __restrict__ sizes, uint32_t g
     }
 }
 
-template <int FMT, int TW, int TM, int WW, int WM, int EPI>
-int launch_gemm(const GemmParams& p, uint32_t max_m_tiles, hipStream_t s) {
+template <int FMT, int TW, int TM, int WW, int WM, int EPI, bool FAST>
+int launch_gemm_impl(const GemmParams& p, uint32_t max_m_tiles, hipStream_t s) {
     constexpr int kScaleDw = FMT == CMX_FMT_E2M1 ? 2 : 1;
     constexpr size_t smem = 2 * ((TW + TM) * kSlabBytes + (TW + TM) * 4 * kScaleDw);
-    auto kfn = mx_gemm_kernel<FMT, TW, TM, WW, WM, EPI>;
+    auto kfn = mx_gemm_kernel<FMT, TW, TM, WW, WM, EPI, FAST>;
     static bool attr_set = false;
     if (!attr_set) {
         CMX_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kfn), hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -457,30 +741,75 @@ int launch_gemm(const GemmParams& p, uint32_t max_m_tiles, hipStream_t s) {
     }
     const uint64_t tiles = (uint64_t)max_m_tiles * p.w_tiles;
     CMX_REQUIRE(tiles > 0 && tiles < (1ull << 31), "tile count out of range");
-    hipLaunchKernelGGL(kfn, dim3((uint32_t)tiles), dim3(kThreads), smem, s, p);
+    hipLaunchKernelGGL(kfn, dim3((uint32_t)tiles), dim3(64 * WW * WM), smem, s, p);
     CMX_LAUNCH_CHECK();
     return CMX_OK;
 }
 
+template <int FMT, int TW, int TM, int WW, int WM, int EPI>
+int launch_gemm_dl(const GemmParams& p, uint32_t max_m_tiles, hipStream_t s) {
+    constexpr int kScaleDw = FMT == CMX_FMT_E2M1 ? 2 : 1;
+    constexpr size_t smem = 2 * (TW + TM) * kSlabBytes + 2 * (TW + TM) * kScaleDw * 4;
+    auto kfn = mx_gemm_dl_kernel<FMT, TW, TM, WW, WM, EPI>;
+    static bool attr_set = false;
+    if (!attr_set) {
+        CMX_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kfn), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                    (int)smem));
+        attr_set = true;
+    }
+    const uint64_t tiles = (uint64_t)max_m_tiles * p.w_tiles;
+    CMX_REQUIRE(tiles > 0 && tiles < (1ull << 31), "tile count out of range");
+    hipLaunchKernelGGL(kfn, dim3((uint32_t)tiles), dim3(64 * WW * WM), smem, s, p);
+    CMX_LAUNCH_CHECK();
+    return CMX_OK;
+}
+
+bool g_disable_dl = false;   // tuning/test hook: force the register-staged kernels
+
+template <int FMT, int TW, int TM, int WW, int WM, int EPI>
+int launch_gemm(const GemmParams& p, uint32_t max_m_tiles, hipStream_t s) {
+    // streaming kernel: whole 128-element scale groups, dword-aligned scale rows, four wavefronts
+    if constexpr (TW % (8 * WW * WM) == 0 && TM % (8 * WW * WM) == 0 && TW % 64 == 0 && TM % 64 == 0) {
+        if (!g_disable_dl && p.scale_vec && p.kbytes % kSlabBytes == 0)
+            return launch_gemm_dl<FMT, TW, TM, WW, WM, EPI>(p, max_m_tiles, s);
+    }
+    const bool fast = p.scale_vec && (p.kbytes % kSlabBytes == 0);
+    if (fast) return launch_gemm_impl<FMT, TW, TM, WW, WM, EPI, true>(p, max_m_tiles, s);
+    return launch_gemm_impl<FMT, TW, TM, WW, WM, EPI, false>(p, max_m_tiles, s);
+}
+
 struct TileChoice {
-    int tw, tm;
+    int tw, tm, waves;
 };
 
-int g_force_tile = 0;   // test/tuning hook: 0 = heuristic, else tw*1000 + tm
+TileChoice g_force_tile = {0, 0, 0};   // test/tuning hook: tw == 0 -> heuristic
 
 TileChoice choose_tile(uint32_t m_hint, uint32_t n) {
-    if (g_force_tile) return {g_force_tile / 1000, g_force_tile % 1000};
-    if (m_hint <= 64) return {256, 64};
-    if (m_hint <= 128) return {256, 128};
-    return {256, 256};
+    if (g_force_tile.tw) return g_force_tile;
+    if (m_hint <= 64) return {256, 64, 4};
+    if (m_hint <= 128) return {256, 128, 8};
+    return {256, 256, 8};
+}
+
+// Eight-wavefront shapes exist only as streaming kernels; when a problem is not eligible for
+// streaming (ragged K, unaligned scale rows) the four-wavefront register-staged kernel of the same
+// tile takes over.
+template <int FMT, int TW, int TM, int EPI>
+int launch_tile(const GemmParams& p, int waves, uint32_t max_m_tiles, hipStream_t s) {
+    const bool stream_ok = !g_disable_dl && p.scale_vec && p.kbytes % kSlabBytes == 0;
+    if constexpr (TM >= 128) {
+        if (waves == 8 && stream_ok) return launch_gemm_dl<FMT, TW, TM, 2, 4, EPI>(p, max_m_tiles, s);
+    }
+    constexpr int WW = TM >= 128 ? 2 : 4, WM = TM >= 128 ? 2 : 1;
+    return launch_gemm<FMT, TW, TM, WW, WM, EPI>(p, max_m_tiles, s);
 }
 
 template <int FMT, int EPI>
 int dispatch_tile(const GemmParams& p, TileChoice t, uint32_t max_m_tiles, hipStream_t s) {
-    if (t.tw == 256 && t.tm == 256) return launch_gemm<FMT, 256, 256, 2, 2, EPI>(p, max_m_tiles, s);
-    if (t.tw == 256 && t.tm == 128) return launch_gemm<FMT, 256, 128, 2, 2, EPI>(p, max_m_tiles, s);
-    if (t.tw == 256 && t.tm == 64) return launch_gemm<FMT, 256, 64, 4, 1, EPI>(p, max_m_tiles, s);
-    if (t.tw == 128 && t.tm == 128) return launch_gemm<FMT, 128, 128, 2, 2, EPI>(p, max_m_tiles, s);
+    if (t.tw == 256 && t.tm == 256) return launch_tile<FMT, 256, 256, EPI>(p, t.waves, max_m_tiles, s);
+    if (t.tw == 256 && t.tm == 128) return launch_tile<FMT, 256, 128, EPI>(p, t.waves, max_m_tiles, s);
+    if (t.tw == 256 && t.tm == 64) return launch_tile<FMT, 256, 64, EPI>(p, t.waves, max_m_tiles, s);
+    if (t.tw == 128 && t.tm == 128) return launch_tile<FMT, 128, 128, EPI>(p, t.waves, max_m_tiles, s);
     set_error("unsupported tile shape");
     return CMX_EINVAL;
 }
@@ -506,8 +835,14 @@ bool scales_dword_aligned(const void* as, uint32_t ld_as, const void* ws, uint32
 
 }  // namespace cmx
 
-extern "C" int cmx_debug_force_tile(int tw, int tm) {
-    cmx::g_force_tile = (tw > 0 && tm > 0) ? tw * 1000 + tm : 0;
+extern "C" int cmx_debug_disable_streaming(int off) {
+    cmx::g_disable_dl = off != 0;
+    return CMX_OK;
+}
+
+// tuning/test hook: pin the tile shape and wavefront count (tw = 0 restores the heuristic)
+extern "C" int cmx_debug_force_tile(int tw, int tm, int waves) {
+    cmx::g_force_tile = (tw > 0 && tm > 0) ? cmx::TileChoice{tw, tm, waves > 0 ? waves : 4} : cmx::TileChoice{0, 0, 0};
     return CMX_OK;
 }
 
@@ -526,6 +861,7 @@ extern "C" int cmx_mx_gemm(const uint8_t* a, uint32_t lda, const uint8_t* a_scal
     p.m = m; p.n = n; p.kbytes = fmt == CMX_FMT_E2M1 ? k / 2 : k; p.kblocks = k / 32;
     p.groups = 1; p.out_type = out_type;
     p.scale_vec = scales_dword_aligned(a_scale, ld_as, b_scale, ld_bs);
+    CMX_REQUIRE((uint64_t)n * ldb < (1ull << 32) && (uint64_t)lda * 256 < (1ull << 32), "operand tile exceeds 32-bit offsets");
     TileChoice t = choose_tile(m, n);
     p.w_tiles = ceil_div(n, t.tw);
     const uint32_t m_tiles = ceil_div(m, t.tm);
@@ -547,6 +883,8 @@ int gmm_common(GemmParams& p, const int32_t* group_sizes, uint32_t groups, uint3
                bool swiglu, hipStream_t s) {
     CMX_REQUIRE(group_sizes && workspace, "null pointer");
     CMX_REQUIRE(groups > 0 && groups <= 65536, "bad group count");
+    CMX_REQUIRE((uint64_t)p.n * p.ldw < (1ull << 32) && (uint64_t)p.lda * 256 < (1ull << 32),
+                "operand tile exceeds 32-bit offsets");
     CMX_REQUIRE((reinterpret_cast<uintptr_t>(workspace) & 3u) == 0, "workspace must be 4-byte aligned");
     // average rows per group steers the tile height
     TileChoice t = choose_tile(ceil_div(m_total, groups), p.n);

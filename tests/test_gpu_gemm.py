@@ -9,7 +9,7 @@ from tests.gpu_util import dev, host, close_bf16
 
 pytestmark = pytest.mark.gpu
 
-TILES = [(256, 256), (256, 128), (256, 64), (128, 128)]
+TILES = [(256, 256, 4), (256, 256, 8), (256, 128, 4), (256, 128, 8), (256, 64, 4), (128, 128, 4)]
 
 
 def _mx(rng, rows, k, fmt="E4M3", std=1.0):
@@ -28,14 +28,14 @@ def _run(aq, asc, bq, bsc, k, fmt="E4M3", out="bf16"):
 def _reset_tile():
     yield
     from catccos_amd import _lib
-    _lib.load().cmx_debug_force_tile(0, 0)
+    _lib.load().cmx_debug_force_tile(0, 0, 0)
 
 
-@pytest.mark.parametrize("tw,tm", TILES)
+@pytest.mark.parametrize("tw,tm,waves", TILES)
 @pytest.mark.parametrize("m,n,k", [(256, 256, 128), (300, 520, 384), (64, 1000, 7168), (1, 64, 32), (513, 257, 96)])
-def test_dense_fp8_vs_oracle(tw, tm, m, n, k):
+def test_dense_fp8_vs_oracle(tw, tm, waves, m, n, k):
     from catccos_amd import _lib
-    _lib.load().cmx_debug_force_tile(tw, tm)
+    _lib.load().cmx_debug_force_tile(tw, tm, waves)
     rng = np.random.default_rng(m * 7 + n * 3 + k)
     aq, asc = _mx(rng, m, k)
     bq, bsc = _mx(rng, n, k)
@@ -72,11 +72,11 @@ def test_one_hot_rows_copy_weight_rows_exactly():
     assert np.array_equal(c, want)
 
 
-@pytest.mark.parametrize("tw,tm", [(256, 256), (256, 128)])
+@pytest.mark.parametrize("tw,tm,waves", [(256, 256, 4), (256, 256, 8), (256, 128, 4)])
 @pytest.mark.parametrize("m,n,k", [(256, 256, 256), (130, 300, 640), (64, 512, 7168)])
-def test_dense_fp4_vs_oracle(tw, tm, m, n, k):
+def test_dense_fp4_vs_oracle(tw, tm, waves, m, n, k):
     from catccos_amd import _lib
-    _lib.load().cmx_debug_force_tile(tw, tm)
+    _lib.load().cmx_debug_force_tile(tw, tm, waves)
     rng = np.random.default_rng(m + n + k)
     aq, asc = O.mx_quant(rng.uniform(-2, 2, (m, k)).astype(np.float32), "E2M1")
     bq, bsc = O.mx_quant(rng.uniform(-2, 2, (n, k)).astype(np.float32), "E2M1")
