@@ -41,7 +41,7 @@ def main() -> int:
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--only", type=str, default="", help="comma list of extras: quant,gemm,ffn,fp4,routing (default all)")
+    ap.add_argument("--only", type=str, default="", help="comma list of extras: quant,gemm,ffn,fp4,routing,copycal (default: all but copycal)")
     ap.add_argument("--no-extras", action="store_true")
     ap.add_argument("--no-cpu", action="store_true")
     args = ap.parse_args()
@@ -127,8 +127,8 @@ def main() -> int:
     cpu = None
     if not args.no_cpu:
         from oracle import mx_oracle as O
-        sample_groups = [i for i in np.argsort(-counts_h)[:2]]
-        cap = 1024
+        sample_groups = [int(i) for i in np.argsort(-counts_h)[:8]]     # the 8 largest experts, up to 2048 rows each
+        cap = 2048
         off = np.concatenate([[0], np.cumsum(counts_h)])
         a_h, as_h = [], []
         cnt = []
@@ -140,7 +140,7 @@ def main() -> int:
         a_h, as_h = np.concatenate(a_h), np.concatenate(as_h)
         w_h = w1[sample_groups].cpu().numpy()
         ws_h = w1s[sample_groups].cpu().numpy()
-        O.gmm1_swiglu_quant(a_h[:64], as_h[:64], w_h, ws_h, [32, 32])        # warm-up
+        O.gmm1_swiglu_quant(a_h[:64], as_h[:64], w_h[:2], ws_h[:2], [32, 32])        # warm-up
         reps = []
         for _ in range(3):
             t0 = time.perf_counter()
@@ -163,6 +163,17 @@ def main() -> int:
     want = set(x for x in args.only.split(",") if x) or {"quant", "gemm", "ffn", "fp4", "routing"}
     if args.no_extras:
         want = set()
+
+    if "copycal" in want:
+        # plain device copy of known size: calibrates the FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run
+        nbytes = 1 << 30
+        src = torch.empty(nbytes, dtype=torch.uint8, device=dev).fill_(1)
+        dst = torch.empty_like(src)
+        tcopy = hip_time(lambda: dst.copy_(src), steps=5, warm=1)
+        extra["copycal"] = {"bytes_read": nbytes, "bytes_written": nbytes, "avg_launch_us": tcopy * 1e6,
+                            "GBs": 2 * nbytes / tcopy / 1e9}
+        log(f"[copy calibration] 1 GiB -> 1 GiB in {tcopy*1e6:.1f} us = {2*nbytes/tcopy/1e9:.0f} GB/s")
+        del src, dst
 
     if "quant" in want:
         M1, K1 = 4096, 7168
