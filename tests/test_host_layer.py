@@ -1,0 +1,119 @@
+"""The C++ plugin layer (CatccosOperator / OperatorRegistry / launch table / driver).
+
+CPU part: the host-only C++ check program and the driver's argument and validation paths, none of
+which reach the GPU.  GPU part: the driver end to end on .bin files written from seeded inputs, its
+output files compared with the oracle the same way the library-level parity tests do.
+"""
+import os
+import subprocess
+
+import numpy as np
+import pytest
+
+from oracle import mx_oracle as O
+from catccos_amd import workloads as W
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HOST = os.path.join(ROOT, "catccos_amd", "host")
+BIN = os.path.join(HOST, "bin")
+
+
+@pytest.fixture(scope="module")
+def host_bin():
+    if not (os.path.exists(os.path.join(BIN, "catccos_mx_run")) and os.path.exists(os.path.join(BIN, "test_host_layer"))):
+        from catccos_amd import build
+        build.build(force=False)
+        subprocess.run(["make", "-C", HOST, "all"], check=True, capture_output=True)
+    return BIN
+
+
+def _run(host_bin, *args, timeout=120):
+    return subprocess.run([os.path.join(host_bin, "catccos_mx_run"), *map(str, args)], capture_output=True, text=True, timeout=timeout)
+
+
+def test_host_checks(host_bin):
+    r = subprocess.run([os.path.join(host_bin, "test_host_layer")], capture_output=True, text=True, timeout=60)
+    assert r.returncode == 0, r.stdout + r.stderr
+    assert "host layer checks: PASS" in r.stdout
+
+
+def test_driver_rejects_before_touching_the_gpu(host_bin):
+    r = _run(host_bin, "a5moe", 4, 7168)
+    assert r.returncode == 1 and "Usage" in r.stderr
+    r = _run(host_bin, "NoSuchOperator", 4, 256, 512)
+    assert r.returncode != 0 and "not found" in r.stdout
+    r = _run(host_bin, "a5moe", 4, 7168 + 128, 4096)                   # K % 256 != 0
+    assert r.returncode != 0 and "Invalid CocTilingParams" in r.stderr
+    r = _run(host_bin, "a5moe", 4, 7168, 4096, "--experts", 4, "--topk", 6)      # topK > experts
+    assert r.returncode != 0 and "Invalid CocTilingParams" in r.stderr
+    r = _run(host_bin, "a5moe", 0, 7168, 4096)
+    assert r.returncode == 1 and "positive uint32" in r.stderr
+    r = _run(host_bin, "a5moe", 4, 7168, 4096, "--m0", 64)
+    assert r.returncode == 1 and "Invalid GMM1 M tile" in r.stderr
+    r = _run(host_bin, "mxqtag", 16, 1, 7168 + 16)                      # columns not a multiple of 32
+    assert r.returncode != 0
+
+
+# ---------------------------------------------------------------------------------------------- GPU
+
+def _write(path, arr):
+    np.ascontiguousarray(arr).tofile(path)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("fmt,ofmt", [("e4m3", "E4M3"), ("e5m2", "E5M2"), ("e2m1", "E2M1")])
+def test_driver_quant(host_bin, tmp_path, fmt, ofmt):
+    rows, cols = 96, 7168
+    x = W.activations_with_outliers(rows, cols, seed=5)
+    _write(tmp_path / "rank_0_input.bin", x)
+    r = _run(host_bin, "MxQuantAllGather", rows, 1, cols, "--data", tmp_path, "--fmt", fmt, "--poison")
+    assert r.returncode == 0, r.stdout + r.stderr
+    assert "[TEST] input rank_size: 1 rank_id:0" in r.stdout and "[CONFIG]" in r.stdout
+    codes, scales = O.mx_quant_bf16(x, ofmt, "lut" if ofmt == "E2M1" else "rne")
+    if ofmt == "E2M1":
+        codes = O.pack_fp4(codes)
+    got = np.fromfile(tmp_path / "rank_0_output.bin", dtype=np.uint8).reshape(codes.shape)
+    got_s = np.fromfile(tmp_path / "rank_0_mxscale.bin", dtype=np.uint8).reshape(scales.shape)
+    assert np.array_equal(got, codes) and np.array_equal(got_s, scales)
+
+
+@pytest.mark.gpu
+def test_driver_mxfp8_matmul(host_bin, tmp_path):
+    m, k, n = 192, 1024, 384
+    rng = np.random.default_rng(11)
+    aq, asc = O.mx_quant(O.bf16_round(rng.standard_normal((m, k)).astype(np.float32)), "E4M3", "rne")
+    bq, bsc = O.mx_quant(O.bf16_round(rng.standard_normal((n, k)).astype(np.float32) / np.sqrt(k)), "E4M3", "lut")
+    for stem, arr in (("a", aq), ("b", bq), ("a_scale", asc), ("b_scale", bsc)):
+        _write(tmp_path / f"rank_0_{stem}.bin", arr)
+    r = _run(host_bin, "a5mxfp8mmrs", m, k, n, "--data", tmp_path)
+    assert r.returncode == 0, r.stdout + r.stderr
+    got = np.fromfile(tmp_path / "output.bin", dtype=np.uint16).reshape(m, n)
+    gold = O.mx_gemm_f32(aq, asc, bq, bsc)
+    assert np.allclose(O.bf16_bits_to_f32(got), gold, rtol=1e-2, atol=1e-2)
+
+
+@pytest.mark.gpu
+def test_driver_ffn(host_bin, tmp_path):
+    tokens, k, n, experts, top_k = 64, 512, 1024, 8, 4
+    rng = np.random.default_rng(3)
+    x = W.normal_bf16((tokens, k), 3)
+    idx, p = W.softmax_topk_routing(tokens, experts, top_k, 4)
+    w1 = [O.mx_quant(O.bf16_round(rng.standard_normal((n, k)).astype(np.float32) / np.sqrt(k)), "E4M3", "lut") for _ in range(experts)]
+    w2 = [O.mx_quant(O.bf16_round(rng.standard_normal((k, n // 2)).astype(np.float32) / np.sqrt(n // 2)), "E4M3", "lut") for _ in range(experts)]
+    w1q, w1s = np.stack([a for a, _ in w1]), np.stack([b for _, b in w1])
+    w2q, w2s = np.stack([a for a, _ in w2]), np.stack([b for _, b in w2])
+    for stem, arr in (("in_routing_matrix_a", x), ("in_gmm_matrix_b", w1q), ("in_gmm_matrix_b2", w2q), ("in_gmm_matrix_b_scale", w1s),
+                      ("in_gmm_matrix_b2_scale", w2s), ("in_routing_expert_idx", idx.astype(np.int32)), ("in_gather_gate_weight", p.astype(np.float32))):
+        _write(tmp_path / f"{stem}_0.bin", arr)
+    r = _run(host_bin, "Ascend950DispatchFFNCombine", tokens, k, n, "--experts", experts, "--topk", top_k, "--data", tmp_path, "--poison",
+             "--repeats", 2)
+    assert r.returncode == 0, r.stdout + r.stderr
+    got = np.fromfile(tmp_path / "output_0.bin", dtype=np.uint16).reshape(tokens, k)
+    gold = O.bf16_bits_to_f32(O.moe_ffn(x, idx, p, w1q, w1s, w2q, w2s))
+    ok, err, eb = O.verify_bf16(got, gold, 1 << 20)
+    diff = np.abs(O.bf16_bits_to_f32(got) - gold)
+    assert (diff > 1e-2 + 1e-2 * np.abs(gold)).sum() <= got.size // 1000 and eb <= 2.0 ** -7, (err, eb)
+    # a missing input file is an error, not a silent default
+    os.remove(tmp_path / "in_gather_gate_weight_0.bin")
+    r = _run(host_bin, "a5moe", tokens, k, n, "--experts", experts, "--topk", top_k, "--data", tmp_path)
+    assert r.returncode != 0 and "ERROR" in r.stderr
