@@ -444,13 +444,9 @@ __global__ __launch_bounds__(64 * WW * WM) void mx_gemm_kernel(const GemmParams 
     __syncthreads();
     // steady state is branch free: prefetch slab s+1, consume slab s, refill the other stage
     for (uint32_t s = 0; s + 1 < nslab; ++s) {
-#if !(defined(CMX_DBG_SKIP) && (CMX_DBG_SKIP & 1))
         load_global(s + 1);
-#endif
         __builtin_amdgcn_sched_barrier(0);
-#if !(defined(CMX_DBG_SKIP) && (CMX_DBG_SKIP & 2))
         compute(s & 1u);
-#endif
         // Keep the LDS refill (which waits for the global loads) behind the MFMAs of this slab: without
         // a use of the accumulators here the compiler sinks the MFMAs below the refill and the barrier,
         // which exposes the whole global-load latency every iteration.
@@ -459,9 +455,7 @@ __global__ __launch_bounds__(64 * WW * WM) void mx_gemm_kernel(const GemmParams 
 #pragma unroll
             for (int j = 0; j < FM; ++j) asm volatile("" ::"a"(acc[i][j][0]) : "memory");
         __builtin_amdgcn_sched_barrier(0);
-#if !(defined(CMX_DBG_SKIP) && (CMX_DBG_SKIP & 4))
         store_lds((s + 1) & 1u);
-#endif
         __syncthreads();
     }
     compute((nslab - 1) & 1u);
@@ -656,20 +650,15 @@ __global__ __launch_bounds__(64 * WW * WM) void mx_gemm_dl_kernel(const GemmPara
     for (uint32_t s = 0; s < nslab; ++s) {
 #pragma unroll
         for (int h = 0; h < kSub; ++h) {
-#ifndef CMX_DBG_SKIP
-#define CMX_DBG_SKIP 0
-#endif
             if (h + 1 < kSub) {
-                if (!(CMX_DBG_SKIP & 8)) read_frags(s, h + 1, (h + 1) & 1);
+                read_frags(s, h + 1, (h + 1) & 1);
             } else {
                 // slot s&1 is drained by this wavefront one step early: refill point
-                if (!(CMX_DBG_SKIP & 16)) {
                 CMX_WAIT_ALL();                 // own fragment reads of slab s and own loads of slab s+1 are done
                 __syncthreads();                // ... and everyone else's
-                }
-                if (!(CMX_DBG_SKIP & 1)) issue_slab(s + 2);
-                if (!(CMX_DBG_SKIP & 8)) read_frags(s + 1, 0, 0);
-                if (!(CMX_DBG_SKIP & 8)) read_scales(s + 1, swn, san);
+                issue_slab(s + 2);
+                read_frags(s + 1, 0, 0);
+                read_scales(s + 1, swn, san);
             }
             // One wavefront per SIMD issues in order, so the MFMA pipe idles whenever more than one
             // MFMA time of other instructions sits between two MFMAs: spread the LDS reads and the

@@ -215,13 +215,22 @@ int cmx_ffn_workspace_layout_get(uint32_t m, uint32_t k, uint32_t n, uint32_t lo
                                  cmx_ffn_workspace_layout* layout);
 
 /* ------------------------------------------------------------------------------------------
- * Single-tile probe of the block-scaled MFMA (used by the layout known-answer tests):
- * out fp32 [32, 32] = deq(w)[32 rows, 64 k] . deq(a)[32 rows, 64 k]^T with one E8M0 scale per
- * (row, 32-k block).  w/a: fmt codes [32, 64] (FP4: [32, 32] bytes); ws/as: u8 [32, 2].
- * out[i][j] = sum_k w[i,k] * a[j,k].
+ * Test and tuning hooks (no counterpart in the reference).
+ *
+ * cmx_mfma_raw_probe: one wavefront executes one block-scaled MFMA on caller-supplied registers, so
+ * the operand/scale/accumulator lane layout the GEMM kernels rely on can be pinned by known-answer
+ * tests.  a_regs/b_regs: int32 [64 lanes][8]; sa/sb: int32 [64] (scale VGPR per lane, byte `opsel`
+ * is used for both operands); out: fp32 [64][16] (shape 0: 32x32x64) or [64][4] (shape 1: 16x16x128).
+ *
+ * cmx_debug_force_tile: (tw, tm, waves) overrides the tile heuristic of every later matmul call in
+ * this process so tests can cover every compiled tile shape; tw <= 0 restores the heuristic.
+ * cmx_debug_disable_streaming: non-zero forces the register-staged kernels instead of the
+ * LDS-streaming ones.  Neither hook is thread safe; both return CMX_OK.
  * ---------------------------------------------------------------------------------------- */
-int cmx_mfma_tile_probe(const uint8_t* w, const uint8_t* ws, const uint8_t* a, const uint8_t* as, float* out,
-                        int fmt, cmx_stream_t stream);
+int cmx_mfma_raw_probe(const void* a_regs, const void* b_regs, const int32_t* sa, const int32_t* sb, float* out,
+                       int fmt, int opsel, int shape, cmx_stream_t stream);
+int cmx_debug_force_tile(int tw, int tm, int waves);
+int cmx_debug_disable_streaming(int off);
 
 #ifdef __cplusplus
 }

@@ -1,0 +1,44 @@
+"""The C-ABI library loads without a GPU and exports exactly what include/catccos_mx.h declares."""
+import ctypes
+import os
+import re
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "catccos_mx.h")
+
+
+def _declared():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)          # drop comments
+    text = re.sub(r"//[^\n]*", "", text)
+    names = re.findall(r"\b((?:cmx|catccos_ascend950)_[a-z0-9_]+)\s*\(", text)
+    return sorted(set(names))
+
+
+def test_header_declares_the_expected_surface():
+    names = _declared()
+    for must in ("cmx_mx_quant", "cmx_mx_dequant", "cmx_mx_gemm", "cmx_mx_gmm", "cmx_mx_gmm_swiglu_quant", "cmx_moe_init_routing",
+                 "cmx_quant_scatter", "cmx_moe_token_unpermute", "catccos_ascend950_dispatch_ffn_combine",
+                 "catccos_ascend950_dispatch_ffn_combine_workspace_bytes", "catccos_ascend950_symmetric_bytes"):
+        assert must in names
+    assert len(names) >= 25
+
+
+def test_library_exports_every_declared_symbol():
+    from catccos_amd import _lib
+    lib = _lib.load()
+    missing = [n for n in _declared() if not hasattr(lib, n)]
+    assert not missing, missing
+    # the ctypes table of the Python front end covers the same set
+    assert sorted(_lib.SIGNATURES) == _declared()
+
+
+def test_host_only_entry_points_work_without_a_gpu():
+    from catccos_amd import _lib
+    lib = _lib.load()
+    assert lib.cmx_version() >= 1
+    assert lib.catccos_ascend950_symmetric_bytes() == 1004 * 1024 * 1024
+    assert lib.cmx_packed_row_bytes(7168) == 7168 + 224
+    # a bad argument is reported through the error string, not a crash
+    rc = lib.cmx_mx_quant(None, 0, None, 0, None, 0, 1, 33, 0, 0, None)
+    assert rc != 0 and lib.cmx_last_error()
