@@ -140,6 +140,92 @@ __global__ __launch_bounds__(kThreads) void mx_quant_kernel(const uint16_t* __re
     }
 }
 
+// ---- fast path: RNE 8-bit formats, cols % 32 == 0, 16-byte aligned rows ------------------------
+// Same lane split (four lanes per block, one 16-byte load each) but laid out so that no lane ever
+// divides: a workgroup owns 64 consecutive blocks of four consecutive rows, one row per unroll step.
+// The arithmetic stays on packed 16-bit integers until the final cast: amax and the clamp to
+// +-max_normal * 2^e work on sign-cleared bf16 bit patterns (unsigned order == magnitude order), and
+// v_cvt_scalef32_pk_{fp8,bf8}_bf16 divides by 2^e and rounds to nearest even in one instruction.
+// Each lane of a quad then stores the scale byte of one of the four rows.
+typedef unsigned short v2u16 __attribute__((ext_vector_type(2)));
+typedef short v2i16 __attribute__((ext_vector_type(2)));
+typedef __bf16 v2bf16 __attribute__((ext_vector_type(2)));
+
+constexpr int kFastRows = 4;
+
+__device__ __forceinline__ uint32_t pk_max_u16(uint32_t a, uint32_t b) {
+    return __builtin_bit_cast(uint32_t, __builtin_elementwise_max(__builtin_bit_cast(v2u16, a), __builtin_bit_cast(v2u16, b)));
+}
+__device__ __forceinline__ uint32_t pk_min_u16(uint32_t a, uint32_t b) {
+    return __builtin_bit_cast(uint32_t, __builtin_elementwise_min(__builtin_bit_cast(v2u16, a), __builtin_bit_cast(v2u16, b)));
+}
+
+template <int FMT>
+__device__ __forceinline__ uint32_t cvt_scaled_pk4(uint32_t d0, uint32_t d1, float scale) {
+    v2i16 o = {0, 0};
+    if constexpr (FMT == CMX_FMT_E4M3) {
+        o = __builtin_amdgcn_cvt_scalef32_pk_fp8_bf16(o, __builtin_bit_cast(v2bf16, d0), scale, false);
+        o = __builtin_amdgcn_cvt_scalef32_pk_fp8_bf16(o, __builtin_bit_cast(v2bf16, d1), scale, true);
+    } else {
+        o = __builtin_amdgcn_cvt_scalef32_pk_bf8_bf16(o, __builtin_bit_cast(v2bf16, d0), scale, false);
+        o = __builtin_amdgcn_cvt_scalef32_pk_bf8_bf16(o, __builtin_bit_cast(v2bf16, d1), scale, true);
+    }
+    return __builtin_bit_cast(uint32_t, o);
+}
+
+template <int FMT>
+__global__ __launch_bounds__(kThreads) void mx_quant_rne8_kernel(const uint8_t* __restrict__ x, uint32_t ld_x_bytes,
+                                                                 uint8_t* __restrict__ codes, uint32_t ld_codes,
+                                                                 uint8_t* __restrict__ scales, uint32_t ld_scales,
+                                                                 uint32_t rows, uint32_t nb) {
+    constexpr int emax = FMT == CMX_FMT_E4M3 ? kEmaxE4M3 : kEmaxE5M2;
+    constexpr uint32_t lim_mant = FMT == CMX_FMT_E4M3 ? 0x60u : 0x60u;   // 448 = 1.75 * 2^8, 57344 = 1.75 * 2^15
+    const uint32_t q = threadIdx.x & 3u;
+    const uint32_t kb = blockIdx.x * kBlocksPerIter + (threadIdx.x >> 2);
+    const uint32_t row0 = blockIdx.y * kFastRows;
+    if (kb >= nb) return;                                  // whole quads leave together
+    const uint32_t in_off = kb * 64u + q * 16u;            // bytes inside the row
+    const uint32_t out_off = kb * 32u + q * 8u;
+
+    uint4 raw[kFastRows];
+#pragma unroll
+    for (int u = 0; u < kFastRows; ++u) {
+        const uint32_t row = row0 + u;
+        raw[u] = make_uint4(0, 0, 0, 0);
+        if (row < rows) raw[u] = *reinterpret_cast<const uint4*>(x + (size_t)row * ld_x_bytes + in_off);
+    }
+    int my_e = 0;
+#pragma unroll
+    for (int u = 0; u < kFastRows; ++u) {
+        const uint32_t row = row0 + u;
+        const uint32_t d[4] = {raw[u].x, raw[u].y, raw[u].z, raw[u].w};
+        uint32_t a[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) a[i] = d[i] & 0x7FFF7FFFu;
+        uint32_t m = pk_max_u16(pk_max_u16(a[0], a[1]), pk_max_u16(a[2], a[3]));
+        m = pk_max_u16(m, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)m, 0xB1, 0xF, 0xF, true));
+        m = pk_max_u16(m, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)m, 0x4E, 0xF, 0xF, true));
+        const uint32_t amax = max(m & 0xFFFFu, m >> 16);
+        const int e = block_exp_from_bf16_amax(amax, emax);
+        // clamp magnitudes to max_normal * 2^e (bit pattern: exponent e + emax + 127, mantissa 1.75)
+        const uint32_t lim = (((uint32_t)(e + emax + 127) << 7) | lim_mant) * 0x10001u;
+        const float scale = __uint_as_float((uint32_t)(e + 127) << 23);
+        uint32_t c[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) c[i] = pk_min_u16(a[i], lim) | (d[i] & 0x80008000u);
+        const uint32_t w0 = cvt_scaled_pk4<FMT>(c[0], c[1], scale);
+        const uint32_t w1 = cvt_scaled_pk4<FMT>(c[2], c[3], scale);
+        if (row < rows) *reinterpret_cast<uint2*>(codes + (size_t)row * ld_codes + out_off) = make_uint2(w0, w1);
+        my_e = (int)q == u ? e : my_e;
+    }
+    const uint32_t srow = row0 + q;
+    if (srow < rows) {
+        uint8_t* sp = scales + (size_t)srow * ld_scales;
+        sp[kb] = (uint8_t)(my_e + 127);
+        if (kb == nb - 1 && (nb & 1u)) sp[nb] = 127;       // pad the scale row to an even count with 1.0
+    }
+}
+
 __global__ void mx_dequant_kernel(const uint8_t* __restrict__ codes, uint32_t ld_codes,
                                   const uint8_t* __restrict__ scales, uint32_t ld_scales, float* __restrict__ out,
                                   uint32_t ld_out, uint32_t rows, uint32_t cols, int fmt) {
@@ -204,6 +290,20 @@ extern "C" int cmx_mx_quant(const void* x, uint32_t ld_x, uint8_t* codes, uint32
     hipStream_t s = static_cast<hipStream_t>(stream);
     const uint16_t* xp = static_cast<const uint16_t*>(x);
     const bool lut = round_mode == CMX_ROUND_LUT;
+    const bool fast = !lut && fmt != CMX_FMT_E2M1 && cols % 32 == 0 && vec_in && vec_out &&
+                      (uint64_t)ld_x * 2 < (1ull << 32) && ceil_div(rows, kFastRows) <= 65535u;
+    if (fast) {
+        dim3 fgrid(ceil_div(nb, kBlocksPerIter), ceil_div(rows, kFastRows));
+        const uint8_t* xb = static_cast<const uint8_t*>(x);
+        if (fmt == CMX_FMT_E4M3)
+            hipLaunchKernelGGL((mx_quant_rne8_kernel<CMX_FMT_E4M3>), fgrid, dim3(kThreads), 0, s, xb, ld_x * 2, codes, ld_codes,
+                               scales, ld_scales, rows, nb);
+        else
+            hipLaunchKernelGGL((mx_quant_rne8_kernel<CMX_FMT_E5M2>), fgrid, dim3(kThreads), 0, s, xb, ld_x * 2, codes, ld_codes,
+                               scales, ld_scales, rows, nb);
+        CMX_LAUNCH_CHECK();
+        return CMX_OK;
+    }
     switch (fmt) {
         case CMX_FMT_E4M3:
             return launch_quant<CMX_FMT_E4M3>(lut, grid, s, xp, ld_x, codes, ld_codes, scales, ld_scales, rows, cols, nb,
