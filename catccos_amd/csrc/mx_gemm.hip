@@ -698,6 +698,8 @@ __global__ __launch_bounds__(64 * WW * WM) void mx_gemm_dl_kernel(const GemmPara
     epilogue<TW, TM, WW, WM, EPI, FW, FM>(p, tc, acc, ww, wm, lane);
 }
 
+#include "mx_gemm_pipe.h"
+
 // Row offsets and m-tile prefix of the groups (one workgroup).
 __global__ void gmm_prepare_kernel(const int32_t* __restrict__ sizes, uint32_t groups, uint32_t tile_m,
                                    int32_t* __restrict__ row_off, int32_t* __restrict__ tile_pref) {
@@ -753,6 +755,23 @@ int launch_gemm_dl(const GemmParams& p, uint32_t max_m_tiles, hipStream_t s) {
     return CMX_OK;
 }
 
+template <int FMT, int EPI>
+int launch_gemm_pipe(const GemmParams& p, uint32_t max_m_tiles, hipStream_t s) {
+    constexpr size_t smem = 2 * 512 * kSlabBytes + 2 * 512 * 4;
+    auto kfn = mx_gemm_pipe_kernel<FMT, EPI>;
+    static bool attr_set = false;
+    if (!attr_set) {
+        CMX_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kfn), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                    (int)smem));
+        attr_set = true;
+    }
+    const uint64_t tiles = (uint64_t)max_m_tiles * p.w_tiles;
+    CMX_REQUIRE(tiles > 0 && tiles < (1ull << 31), "tile count out of range");
+    hipLaunchKernelGGL(kfn, dim3((uint32_t)tiles), dim3(256), smem, s, p);
+    CMX_LAUNCH_CHECK();
+    return CMX_OK;
+}
+
 bool g_disable_dl = false;   // tuning/test hook: force the register-staged kernels
 
 template <int FMT, int TW, int TM, int WW, int WM, int EPI>
@@ -788,6 +807,9 @@ int launch_tile(const GemmParams& p, int waves, uint32_t max_m_tiles, hipStream_
     const bool stream_ok = !g_disable_dl && p.scale_vec && p.kbytes % kSlabBytes == 0;
     if constexpr (TM >= 128) {
         if (waves == 8 && stream_ok) return launch_gemm_dl<FMT, TW, TM, 2, 4, EPI>(p, max_m_tiles, s);
+    }
+    if constexpr (TW == 256 && TM == 256 && FMT != CMX_FMT_E2M1) {
+        if (waves == 4 && stream_ok && p.kbytes % (2 * kSlabBytes) == 0) return launch_gemm_pipe<FMT, EPI>(p, max_m_tiles, s);
     }
     constexpr int WW = TM >= 128 ? 2 : 4, WM = TM >= 128 ? 2 : 1;
     return launch_gemm<FMT, TW, TM, WW, WM, EPI>(p, max_m_tiles, s);

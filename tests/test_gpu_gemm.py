@@ -32,7 +32,7 @@ def _reset_tile():
 
 
 @pytest.mark.parametrize("tw,tm,waves", TILES)
-@pytest.mark.parametrize("m,n,k", [(256, 256, 128), (300, 520, 384), (64, 1000, 7168), (1, 64, 32), (513, 257, 96)])
+@pytest.mark.parametrize("m,n,k", [(256, 256, 128), (300, 520, 384), (64, 1000, 7168), (1, 64, 32), (513, 257, 96), (300, 520, 256), (513, 700, 1024)])
 def test_dense_fp8_vs_oracle(tw, tm, waves, m, n, k):
     from catccos_amd import _lib
     _lib.load().cmx_debug_force_tile(tw, tm, waves)
