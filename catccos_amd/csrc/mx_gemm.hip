@@ -755,10 +755,10 @@ int launch_gemm_dl(const GemmParams& p, uint32_t max_m_tiles, hipStream_t s) {
     return CMX_OK;
 }
 
-template <int FMT, int EPI>
+template <int FMT, int EPI, int TM, int WW, int WM, int NSLOT>
 int launch_gemm_pipe(const GemmParams& p, uint32_t max_m_tiles, hipStream_t s) {
-    constexpr size_t smem = 2 * 512 * kSlabBytes + 2 * 512 * 4;
-    auto kfn = mx_gemm_pipe_kernel<FMT, EPI>;
+    constexpr size_t smem = NSLOT * (256 + TM) * (kSlabBytes + 4);
+    auto kfn = mx_gemm_pipe_kernel<FMT, EPI, TM, WW, WM, NSLOT>;
     static bool attr_set = false;
     if (!attr_set) {
         CMX_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kfn), hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -792,11 +792,15 @@ struct TileChoice {
 
 TileChoice g_force_tile = {0, 0, 0};   // test/tuning hook: tw == 0 -> heuristic
 
-TileChoice choose_tile(uint32_t m_hint, uint32_t n) {
+// waves: at 256 x 256 "4" and "5" select the hand-scheduled kernel in its 2 x 2 and 4 x 1 wavefront layouts
+// when the problem is eligible for it (8-bit elements, an even number of 128-byte K slabs).  Grouped
+// problems take 4 x 1, whose cost follows the valid rows of a ragged group's last tile; FP4 takes the
+// eight-wavefront streaming kernel.
+TileChoice choose_tile(uint32_t m_hint, uint32_t n, int fmt, bool grouped) {
     if (g_force_tile.tw) return g_force_tile;
     if (m_hint <= 64) return {256, 64, 4};
     if (m_hint <= 128) return {256, 128, 8};
-    return {256, 256, 8};
+    return {256, 256, fmt == CMX_FMT_E2M1 ? 8 : (grouped ? 5 : 4)};
 }
 
 // Eight-wavefront shapes exist only as streaming kernels; when a problem is not eligible for
@@ -805,11 +809,16 @@ TileChoice choose_tile(uint32_t m_hint, uint32_t n) {
 template <int FMT, int TW, int TM, int EPI>
 int launch_tile(const GemmParams& p, int waves, uint32_t max_m_tiles, hipStream_t s) {
     const bool stream_ok = !g_disable_dl && p.scale_vec && p.kbytes % kSlabBytes == 0;
-    if constexpr (TM >= 128) {
-        if (waves == 8 && stream_ok) return launch_gemm_dl<FMT, TW, TM, 2, 4, EPI>(p, max_m_tiles, s);
-    }
     if constexpr (TW == 256 && TM == 256 && FMT != CMX_FMT_E2M1) {
-        if (waves == 4 && stream_ok && p.kbytes % (2 * kSlabBytes) == 0) return launch_gemm_pipe<FMT, EPI>(p, max_m_tiles, s);
+        if (waves == 4 && stream_ok && p.kbytes % (2 * kSlabBytes) == 0) return launch_gemm_pipe<FMT, EPI, 256, 2, 2, 2>(p, max_m_tiles, s);
+        if (waves == 5 && stream_ok && p.kbytes % (2 * kSlabBytes) == 0) return launch_gemm_pipe<FMT, EPI, 256, 4, 1, 2>(p, max_m_tiles, s);
+    }
+    if constexpr (TW == 256 && TM == 128 && FMT != CMX_FMT_E2M1) {
+        if (waves == 5 && stream_ok) return launch_gemm_pipe<FMT, EPI, 128, 4, 1, 3>(p, max_m_tiles, s);
+    }
+    if constexpr (TM >= 128) {
+        // the four-wavefront streaming kernel of the 256 x 256 tile runs out of registers: eight there
+        if ((waves == 8 || (TW == 256 && TM == 256)) && stream_ok) return launch_gemm_dl<FMT, TW, TM, 2, 4, EPI>(p, max_m_tiles, s);
     }
     constexpr int WW = TM >= 128 ? 2 : 4, WM = TM >= 128 ? 2 : 1;
     return launch_gemm<FMT, TW, TM, WW, WM, EPI>(p, max_m_tiles, s);
@@ -873,7 +882,7 @@ extern "C" int cmx_mx_gemm(const uint8_t* a, uint32_t lda, const uint8_t* a_scal
     p.groups = 1; p.out_type = out_type;
     p.scale_vec = scales_dword_aligned(a_scale, ld_as, b_scale, ld_bs);
     CMX_REQUIRE((uint64_t)n * ldb < (1ull << 32) && (uint64_t)lda * 256 < (1ull << 32), "operand tile exceeds 32-bit offsets");
-    TileChoice t = choose_tile(m, n);
+    TileChoice t = choose_tile(m, n, fmt, false);
     p.w_tiles = ceil_div(n, t.tw);
     const uint32_t m_tiles = ceil_div(m, t.tm);
     hipStream_t s = static_cast<hipStream_t>(stream);
@@ -898,7 +907,7 @@ int gmm_common(GemmParams& p, const int32_t* group_sizes, uint32_t groups, uint3
                 "operand tile exceeds 32-bit offsets");
     CMX_REQUIRE((reinterpret_cast<uintptr_t>(workspace) & 3u) == 0, "workspace must be 4-byte aligned");
     // average rows per group steers the tile height
-    TileChoice t = choose_tile(ceil_div(m_total, groups), p.n);
+    TileChoice t = choose_tile(ceil_div(m_total, groups), p.n, fmt, true);
     int32_t* row_off = static_cast<int32_t*>(workspace);
     int32_t* tile_pref = row_off + (groups + 1);
     hipLaunchKernelGGL(gmm_prepare_kernel, dim3(1), dim3(256), groups * sizeof(int32_t), s, group_sizes, groups,

@@ -9,12 +9,15 @@
 // a fixed sequence of single-instruction asm statements (their order is kept) with hand-placed
 // s_waitcnt; the compiler still allocates the registers.
 //
-// One slab = 128 bytes of K = two MFMA steps.  Per slab and wavefront:
-//   step 0: 16 MFMAs on fragment set 0; behind the first 8, the 16 reads of fragment set 1 (second
-//           half of the slab); then wait for the own loads of slab s+1 and the own reads of slab s,
-//           barrier (slot s is now free and slab s+1 is visible to everyone);
-//   step 1: 16 MFMAs on fragment set 1; behind them the 16+2 LDS-DMA loads of slab s+2 into the
-//           freed slot, the 16 reads of fragment set 0 from slab s+1 and its 8 scale dwords.
+// One slab = 128 bytes of K = two MFMA steps.  Per slab s (ring slot s%2) and wavefront:
+//   step 0: 16 MFMAs on fragment set 0.  Behind the first 8 go the 16 reads of fragment set 1 (second half
+//           of the slab); after MFMA 8 those reads have landed, and a first barrier says that everybody is
+//           done with the slot, so the loads of slab s+2 into it start right away (7 behind the remaining
+//           MFMAs).  The step ends with the wait for the own loads of slab s+1 (the 7 just issued may stay in
+//           flight) and a second barrier that makes slab s+1 visible to all.
+//   step 1: 16 MFMAs on fragment set 1.  Behind them the other 9+2 loads of slab s+2, the 16 reads of
+//           fragment set 0 from slab s+1, its 8 scale dwords and their per-half-wave byte shift.
+// A load is thus in flight for 23 to 38 MFMA times before anyone waits for it.
 // Every LDS address is a per-lane base register plus an immediate, every global address a per-lane
 // offset register plus a scalar slab offset: the loop contains no address arithmetic on the VALU.
 #pragma once
@@ -39,13 +42,19 @@ __device__ __forceinline__ uint32_t lds_read_b32(uint32_t addr) {
     asm volatile("ds_read_b32 %0, %1 offset:%2" : "=v"(r) : "v"(addr), "n"(OFF) : "memory");
     return r;
 }
+// lds_dst and soff are wavefront-uniform; readfirstlane makes that visible to the register allocator, which
+// otherwise may hand a vector register to an "s" operand.
 __device__ __forceinline__ void dma_b128(uint32_t lds_dst, uint32_t voff, v4i rsrc, uint32_t soff) {
+    lds_dst = __builtin_amdgcn_readfirstlane(lds_dst);
+    soff = __builtin_amdgcn_readfirstlane(soff);
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
                  :
                  : "s"(lds_dst), "v"(voff), "s"(rsrc), "s"(soff)
                  : "memory");
 }
 __device__ __forceinline__ void dma_b32(uint32_t lds_dst, uint32_t voff, v4i rsrc, uint32_t soff) {
+    lds_dst = __builtin_amdgcn_readfirstlane(lds_dst);
+    soff = __builtin_amdgcn_readfirstlane(soff);
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dword %1, %2, %3 offen lds"
                  :
                  : "s"(lds_dst), "v"(voff), "s"(rsrc), "s"(soff)
@@ -53,47 +62,66 @@ __device__ __forceinline__ void dma_b32(uint32_t lds_dst, uint32_t voff, v4i rsr
 }
 
 // acc += W-fragment x A-fragment with the scale byte pair SEL (0: bytes 0/1 of the slab's dword by
-// half-wave, 2: bytes 2/3) of the shifted scale registers.
-template <int FMT, int SEL>
-__device__ __forceinline__ void mfma_acc(v16f& acc, const v8i& w, const v8i& a, uint32_t sw, uint32_t sa) {
+// half-wave, 2: bytes 2/3) of the shifted scale registers.  With BIT >= 0 the instruction is skipped when
+// that bit of the wavefront-uniform `live` mask is clear; the branch sits inside the statement so that the
+// compiler sees straight-line code and adds nothing between the scheduled instructions.
+#define CMX_PIPE_MFMA(SELHI, EXTRA)                                                                             \
+    if constexpr (BIT < 0)                                                                                      \
+        asm volatile("v_mfma_scale_f32_32x32x64_f8f6f4 %0, %1, %2, %0, %3, %4 op_sel_hi:" SELHI EXTRA           \
+                     : "+a"(acc) : "v"(w), "v"(a), "v"(sw), "v"(sa));                                           \
+    else                                                                                                        \
+        asm volatile("s_bitcmp1_b32 %5, %6\n\ts_cbranch_scc0 .Lskip%=\n\t"                                      \
+                     "v_mfma_scale_f32_32x32x64_f8f6f4 %0, %1, %2, %0, %3, %4 op_sel_hi:" SELHI EXTRA           \
+                     "\n.Lskip%=:"                                                                              \
+                     : "+a"(acc) : "v"(w), "v"(a), "v"(sw), "v"(sa), "s"(live), "n"(BIT < 0 ? 0 : BIT) : "scc")
+template <int FMT, int SEL, int BIT>
+__device__ __forceinline__ void mfma_acc(v16f& acc, const v8i& w, const v8i& a, uint32_t sw, uint32_t sa, uint32_t live) {
     static_assert(SEL == 0 || SEL == 2, "scale byte pair");
     if constexpr (FMT == CMX_FMT_E4M3) {
-        if constexpr (SEL == 0)
-            asm volatile("v_mfma_scale_f32_32x32x64_f8f6f4 %0, %1, %2, %0, %3, %4 op_sel_hi:[0,0,0]"
-                         : "+a"(acc) : "v"(w), "v"(a), "v"(sw), "v"(sa));
-        else
-            asm volatile("v_mfma_scale_f32_32x32x64_f8f6f4 %0, %1, %2, %0, %3, %4 op_sel_hi:[1,1,0]"
-                         : "+a"(acc) : "v"(w), "v"(a), "v"(sw), "v"(sa));
+        if constexpr (SEL == 0) { CMX_PIPE_MFMA("[0,0,0]", ""); } else { CMX_PIPE_MFMA("[1,1,0]", ""); }
     } else {
-        if constexpr (SEL == 0)
-            asm volatile("v_mfma_scale_f32_32x32x64_f8f6f4 %0, %1, %2, %0, %3, %4 op_sel_hi:[0,0,0] cbsz:1 blgp:1"
-                         : "+a"(acc) : "v"(w), "v"(a), "v"(sw), "v"(sa));
-        else
-            asm volatile("v_mfma_scale_f32_32x32x64_f8f6f4 %0, %1, %2, %0, %3, %4 op_sel_hi:[1,1,0] cbsz:1 blgp:1"
-                         : "+a"(acc) : "v"(w), "v"(a), "v"(sw), "v"(sa));
+        if constexpr (SEL == 0) { CMX_PIPE_MFMA("[0,0,0]", " cbsz:1 blgp:1"); } else { CMX_PIPE_MFMA("[1,1,0]", " cbsz:1 blgp:1"); }
     }
 }
+#undef CMX_PIPE_MFMA
 
-// Order in which the 8 fragments (0-3 weights, 4-7 activations) are read = order of first use by the
-// MFMA sequence (weight fragment outer, activation fragment inner).
-__device__ __forceinline__ constexpr int pipe_read_order(int i) {
-    return i == 0 ? 0 : (i <= 4 ? 3 + i : i - 4);
+// MFMA sequence of a step: the operand with more fragments runs in the outer loop (weights on a tie).  The
+// fragments (0..FW-1 weights, FW..FW+FM-1 activations) are read in the order of their first use by it.
+template <int FW, int FM>
+__device__ __forceinline__ constexpr int pipe_read_order(int pos) {
+    if (FM > FW) return pos == 0 ? FW : (pos <= FW ? pos - 1 : pos);          // A0 W0..W(FW-1) A1 A2 ...
+    return pos == 0 ? 0 : (pos <= FM ? FW + pos - 1 : pos - FM);              // W0 A0..A(FM-1) W1 W2 ...
 }
 
 __device__ __forceinline__ v8i join8(const v4i& lo, const v4i& hi) {
     return (v8i){lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
 }
 
-template <int FMT, int EPI>
+// Tile = 256 weight rows x TM activation rows, NSLOT ring slots of one slab each.
+//   TM 256, 2 slots, WW x WM = 2 x 2: every wavefront owns a 128 x 128 corner (least LDS traffic per MFMA;
+//           dense problems).
+//   TM 256, 2 slots, 4 x 1: every wavefront owns 64 weight rows x all activation rows and skips the MFMAs of
+//           the 32-row activation blocks past the tile's last valid row, so the last tile of a ragged group
+//           costs what it holds (grouped problems).
+//   TM 128, 3 slots, 4 x 1: two slabs instead of one in flight behind the one being consumed, for groups
+//           so short that every tile streams its weights from HBM once and the load latency, not the MFMA
+//           rate, sets the pace.
+template <int FMT, int EPI, int TM, int WW, int WM, int NSLOT>
 __global__ __launch_bounds__(256) void mx_gemm_pipe_kernel(const GemmParams p) {
     static_assert(FMT == CMX_FMT_E4M3 || FMT == CMX_FMT_E5M2, "8-bit element formats only");
-    constexpr int TW = 256, TM = 256, WW = 2, WM = 2, NW = 4, FW = 4, FM = 4;
+    static_assert((TM == 256 && NSLOT == 2 && ((WW == 2 && WM == 2) || (WW == 4 && WM == 1))) ||
+                      (TM == 128 && NSLOT == 3 && WW == 4 && WM == 1), "tile / ring / wavefront layout");
+    constexpr int TW = 256, NW = 4, FW = TW / WW / 32, FM = TM / WM / 32, NF = FW + FM;
+    constexpr int kM = FW * FM;                                // MFMAs per step and wavefront (16 or 8)
+    constexpr bool kMOuter = FM > FW;                          // activation fragment in the outer MFMA loop
+    constexpr bool kSkip = WM == 1;
     constexpr int kRows = TW + TM;
-    constexpr int kSlotBytes = kRows * kSlabBytes;            // 64 KiB
-    constexpr int kScaleBase = 2 * kSlotBytes;                // scale ring behind the two tile slots
+    constexpr int kSlotBytes = kRows * kSlabBytes;            // 64 KiB or 48 KiB
+    constexpr int kScaleBase = NSLOT * kSlotBytes;            // scale ring behind the tile slots
     constexpr int kScaleSlotBytes = kRows * 4;
-    constexpr int kTileLoads = kRows / (8 * NW);              // 16 LDS-DMA loads per wavefront and slab
+    constexpr int kTileLoads = kRows / (8 * NW);              // LDS-DMA loads per wavefront and slab (16 or 12)
     constexpr int kWTileLoads = TW / (8 * NW);                // the first 8 fetch weight rows
+    constexpr int kLoadsPerSlab = kTileLoads + 2;             // plus one weight and one activation scale load
 
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t*)smem;
@@ -110,9 +138,6 @@ __global__ __launch_bounds__(256) void mx_gemm_pipe_kernel(const GemmParams p) {
     const uint32_t row0 = __builtin_amdgcn_readfirstlane(tc.row0);
     const uint32_t rows_valid = __builtin_amdgcn_readfirstlane(tc.rows_valid);
 
-#ifndef CMX_PIPE_DBG
-#define CMX_PIPE_DBG 0
-#endif
     const uint8_t* wg = p.w + (size_t)g * p.n * p.ldw;
     const uint8_t* wsg = p.w_scale + (size_t)g * p.n * p.ld_ws;
     const uint8_t* ag = p.a + (size_t)row0 * p.lda;
@@ -143,11 +168,12 @@ __global__ __launch_bounds__(256) void mx_gemm_pipe_kernel(const GemmParams p) {
         const uint32_t cr = (NW * i + wave) * 8 + (lane >> 3);
         const uint32_t logical = swz(cr, lane & 7u);
         goff[i] = (i < kWTileLoads ? wrow_of(cr) * p.ldw : arow_of(cr - TW) * p.lda) + logical * 16;
-        if (CMX_PIPE_DBG & 2) goff[i] = (i < kWTileLoads ? (cr - wt * 0) * p.ldw : (cr - TW) * p.lda) + logical * 16;
     }
-    // scale dwords: this wavefront fetches those of weight rows 64*wave.. and activation rows 64*wave..
+    // scale dwords: this wavefront fetches those of weight rows 64*wave.. and of activation rows 64*(wave mod TM/64)..
+    // (with TM = 128 two wavefronts fetch the same rows to the same place)
+    const uint32_t sa_blk = wave % (TM / 64);
     const uint32_t sgoff_w = wrow_of(64 * wave + lane) * p.ld_ws;
-    const uint32_t sgoff_a = arow_of(64 * wave + lane) * p.ld_as;
+    const uint32_t sgoff_a = arow_of(64 * sa_blk + lane) * p.ld_as;
 
     auto make_rsrc = [](const uint8_t* q) -> v4i {
         const uint64_t v = reinterpret_cast<uint64_t>(q);
@@ -158,18 +184,19 @@ __global__ __launch_bounds__(256) void mx_gemm_pipe_kernel(const GemmParams p) {
         r[3] = 0x00020000;
         return r;
     };
-    const v4i w_rs = make_rsrc((CMX_PIPE_DBG & 2) ? p.w : wg), a_rs = make_rsrc((CMX_PIPE_DBG & 2) ? p.a : ag), ws_rs = make_rsrc(wsg), as_rs = make_rsrc(asg);
+    const v4i w_rs = make_rsrc(wg), a_rs = make_rsrc(ag), ws_rs = make_rsrc(wsg), as_rs = make_rsrc(asg);
 
     const uint32_t nslab = p.kbytes / kSlabBytes;
     const uint32_t dma_base = __builtin_amdgcn_readfirstlane(lds0 + wave * 1024);
     const uint32_t sdma_base = __builtin_amdgcn_readfirstlane(lds0 + kScaleBase + wave * 256);
+    const uint32_t sdma_base_a = __builtin_amdgcn_readfirstlane(lds0 + kScaleBase + TW * 4 + sa_blk * 256);
 
     auto issue_tile_load = [&](int slot, int i, uint32_t koff) {
         dma_b128(dma_base + slot * kSlotBytes + i * (NW * 1024), goff[i], i < kWTileLoads ? w_rs : a_rs, koff);
     };
     auto issue_scale_loads = [&](int slot, uint32_t soff) {
         dma_b32(sdma_base + slot * kScaleSlotBytes, sgoff_w, ws_rs, soff);
-        dma_b32(sdma_base + slot * kScaleSlotBytes + TW * 4, sgoff_a, as_rs, soff);
+        dma_b32(sdma_base_a + slot * kScaleSlotBytes, sgoff_a, as_rs, soff);
     };
     auto clamp_slab = [&](uint32_t slab) -> uint32_t { return slab < nslab ? slab : nslab - 1; };   // past the end: harmless reload
 
@@ -178,9 +205,9 @@ __global__ __launch_bounds__(256) void mx_gemm_pipe_kernel(const GemmParams p) {
     // lane share the low five bits l32, hence the swizzle term
     const uint32_t x = (l32 & 7u) ^ ((l32 >> 3) & 1u);
     const uint32_t w_row_base = EPI == kEpiSwigluQuant ? ww * (TW / 2 / WW) : ww * (TW / WW);
-    uint32_t wb[2][4], ab[2][4];       // [slot][chunk j]
+    uint32_t wb[NSLOT][4], ab[NSLOT][4];       // [slot][chunk j]
 #pragma unroll
-    for (int s = 0; s < 2; ++s)
+    for (int s = 0; s < NSLOT; ++s)
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
             const uint32_t ch = ((lh + 2 * j) ^ x) * 16;
@@ -199,132 +226,221 @@ __global__ __launch_bounds__(256) void mx_gemm_pipe_kernel(const GemmParams p) {
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
 
-    // fragment sets: index 0..3 weights, 4..7 activations; lo = registers 0-3, hi = registers 4-7
-    v4i f0lo[8], f0hi[8], f1lo[8], f1hi[8];
-    uint32_t sraw[8], scur[2][8];      // shifted scales alternate between two sets: a set is rewritten one slab after its last use
+    // fragment sets: index 0..FW-1 weights, FW.. activations; lo = registers 0-3, hi = registers 4-7
+    v4i f0lo[NF], f0hi[NF], f1lo[NF], f1hi[NF];
+    uint32_t sraw[NF], scur[NSLOT][NF];      // shifted scales alternate between two sets: a set is rewritten one slab after its last use
 
-    // weight fragment f sits f*32 rows (SwiGLU: gate fragments 0,1 then their up partners 128 rows on) below the base
-    // read order = order of first use by the MFMA sequence (fw outer, fm inner): W0 A0 A1 A2 A3 W1 W2 W3
-#define CMX_PIPE_WOFF(f) ((EPI == kEpiSwigluQuant ? ((f) < 2 ? (f) * 32 : 128 + ((f) - 2) * 32) : (f) * 32))
-    auto read_frag = [&](auto slot_c, auto step_c, auto idx_c, v4i& lo, v4i& hi) {
-        constexpr int slot = decltype(slot_c)::value, step = decltype(step_c)::value, idx = decltype(idx_c)::value;
-        if constexpr (idx < 4) {
-            constexpr int off = CMX_PIPE_WOFF(idx) * kSlabBytes;
-            lo = lds_read_b128<off>(wb[slot][2 * step]);
-            hi = lds_read_b128<off>(wb[slot][2 * step + 1]);
-        } else {
-            constexpr int off = (idx - 4) * 32 * kSlabBytes;
-            lo = lds_read_b128<off>(ab[slot][2 * step]);
-            hi = lds_read_b128<off>(ab[slot][2 * step + 1]);
-        }
+    // weight fragment f sits f*32 rows (SwiGLU: the gate fragments, then their up partners 128 rows on) below the base
+#define CMX_PIPE_WOFF(f) ((EPI == kEpiSwigluQuant ? ((f) < FW / 2 ? (f) * 32 : TW / 2 + ((f) - FW / 2) * 32) : (f) * 32))
+    // one 16-byte read: r = 2 * position in the read order + half (0: registers 0-3, 1: registers 4-7)
+    auto read_half = [&](auto slot_c, auto step_c, auto r_c, v4i (&flo)[NF], v4i (&fhi)[NF]) {
+        constexpr int slot = decltype(slot_c)::value, step = decltype(step_c)::value, r = decltype(r_c)::value;
+        constexpr int idx = pipe_read_order<FW, FM>(r / 2), half = r % 2;
+        (void)wb, (void)ab;
+        v4i& dst = half ? fhi[idx] : flo[idx];
+        if constexpr (idx < FW) dst = lds_read_b128<CMX_PIPE_WOFF(idx) * kSlabBytes>(wb[slot][2 * step + half]);
+        else dst = lds_read_b128<(idx - FW) * 32 * kSlabBytes>(ab[slot][2 * step + half]);
+    };
+    auto read_frag = [&](auto slot_c, auto step_c, auto idx_c, v4i (&flo)[NF], v4i (&fhi)[NF]) {     // by position in the read order
+        constexpr int pos = decltype(idx_c)::value;
+        read_half(slot_c, step_c, std::integral_constant<int, 2 * pos>{}, flo, fhi);
+        read_half(slot_c, step_c, std::integral_constant<int, 2 * pos + 1>{}, flo, fhi);
     };
     auto read_scale = [&](auto slot_c, auto idx_c) {
         constexpr int slot = decltype(slot_c)::value, idx = decltype(idx_c)::value;
-        if constexpr (idx < 4)
+        if constexpr (idx < FW)
             sraw[idx] = lds_read_b32<slot * kScaleSlotBytes + CMX_PIPE_WOFF(idx) * 4>(swb);
         else
-            sraw[idx] = lds_read_b32<slot * kScaleSlotBytes + (idx - 4) * 32 * 4>(sab);
+            sraw[idx] = lds_read_b32<slot * kScaleSlotBytes + (idx - FW) * 32 * 4>(sab);
     };
 
     using I0 = std::integral_constant<int, 0>;
     using I1 = std::integral_constant<int, 1>;
+    using I2 = std::integral_constant<int, 2>;
 
-    // ---- prologue -------------------------------------------------------------------------------------
+    // ---- prologue: fill the ring, wait for slab 0 -------------------------------------------------------
     {
+        static_for<0, NSLOT>([&](auto sc) {
+            constexpr int slot = decltype(sc)::value;
+            const uint32_t k = clamp_slab(slot);
 #pragma unroll
-        for (int i = 0; i < kTileLoads; ++i) issue_tile_load(0, i, 0);
-        issue_scale_loads(0, 0);
-        const uint32_t k1 = clamp_slab(1);
-#pragma unroll
-        for (int i = 0; i < kTileLoads; ++i) issue_tile_load(1, i, k1 * kSlabBytes);
-        issue_scale_loads(1, k1 * 4);
-        asm volatile("s_waitcnt vmcnt(18)\n\ts_barrier" ::: "memory");      // slab 0 has landed everywhere
-        static_for<0, 8>([&](auto ic) {
-            constexpr int idx = pipe_read_order(decltype(ic)::value);
-            read_frag(I0{}, I0{}, std::integral_constant<int, idx>{}, f0lo[idx], f0hi[idx]);
+            for (int i = 0; i < kTileLoads; ++i) issue_tile_load(slot, i, k * kSlabBytes);
+            issue_scale_loads(slot, k * 4);
         });
-        static_for<0, 8>([&](auto ic) { read_scale(I0{}, ic); });
+        asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"((NSLOT - 1) * kLoadsPerSlab) : "memory");      // slab 0 has landed everywhere
+        static_for<0, NF>([&](auto ic) { read_frag(I0{}, I0{}, ic, f0lo, f0hi); });
+        static_for<0, NF>([&](auto ic) { read_scale(I0{}, ic); });
     }
 
     auto shift_scales = [&](auto set_c) {
         constexpr int set = decltype(set_c)::value;
         (void)scur, (void)sraw, (void)sshift;      // asm operands alone do not make a generic lambda capture
 #pragma unroll
-        for (int i = 0; i < 8; ++i) asm volatile("v_lshrrev_b32 %0, %1, %2" : "=v"(scur[set][i]) : "v"(sshift), "v"(sraw[i]));
+        for (int i = 0; i < NF; ++i) asm volatile("v_lshrrev_b32 %0, %1, %2" : "=v"(scur[set][i]) : "v"(sshift), "v"(sraw[i]));
+        asm volatile("s_nop 1" ::: "memory");      // the next MFMA may be the very next instruction (skipped ones in between)
     };
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
     shift_scales(I0{});
 
-    // one slab; SLOT = ring slot of slab s (compile-time so that every LDS offset is an immediate).
-    // On entry fragment set 0 and the shifted scales of the slab are in registers.
-    constexpr int kEarly = 7;       // tile loads of slab s+2 issued already in step 0, behind the first barrier
-    auto slab_body = [&](auto slot_c, uint32_t s) {
+    // activation blocks of 32 rows that hold valid rows (4 x 1 layout: the others are skipped)
+    const uint32_t live = __builtin_amdgcn_readfirstlane((1u << ((rows_valid + 31) / 32)) - 1u);   // bit fm: block has valid rows
+    auto step_mfma = [&](auto sel_c, auto i_c, v4i (&flo)[NF], v4i (&fhi)[NF], auto set_c) {
+        constexpr int sel = decltype(sel_c)::value, i = decltype(i_c)::value, set = decltype(set_c)::value;
+        constexpr int fw = kMOuter ? i % FW : i / FM, fm = kMOuter ? i / FW : i % FM;
+        (void)scur, (void)acc;
+        mfma_acc<FMT, sel, kSkip ? fm : -1>(acc[fw][fm], join8(flo[fw], fhi[fw]), join8(flo[FW + fm], fhi[FW + fm]), scur[set][fw],
+                                            scur[set][FW + fm], live);
+    };
+    // A fragment set stays allocated to the end of the step that consumes it: the reads of the next set must
+    // not be given a register that an MFMA issued a few cycles earlier may still be fetching.
+    auto pin_fragments = [&](v4i (&flo)[NF], v4i (&fhi)[NF]) {
+#pragma unroll
+        for (int i = 0; i < NF; ++i) asm volatile("" ::"v"(flo[i]), "v"(fhi[i]));
+    };
+    // Keep a slab's scale registers allocated to the end of the slab: otherwise the shifts for the next slab
+    // may be given the register of a scale whose last reader is an MFMA issued a few cycles earlier, and
+    // nothing orders that VALU write behind the MFMA's operand fetch.
+    auto pin_scales = [&](auto set_c) {
+        constexpr int set = decltype(set_c)::value;
+        (void)scur;
+#pragma unroll
+        for (int i = 0; i < NF; ++i) asm volatile("" ::"v"(scur[set][i]));
+    };
+    constexpr int kReads = 2 * NF;
+
+    // ---- two-slot ring -------------------------------------------------------------------------------------
+    // One slab; SLOT = ring slot of slab s (compile-time so that every LDS offset is an immediate).  On entry
+    // fragment set 0 and the shifted scales of the slab are in registers.  kR reads go behind each of the first
+    // MFMAs of a step; after MFMA kB1 the last of them has had time to land; kEarly tile loads of slab s+2
+    // are issued already in step 0, behind the first barrier.
+    auto slab_body2 = [&](auto slot_c, uint32_t s) {
         constexpr int slot = decltype(slot_c)::value;
+        constexpr int kR = NF > 8 ? 3 : 2;
+        constexpr int kB1 = (kReads + kR - 1) / kR;
+        constexpr int kEarly = kM - kB1 - 1;
+        constexpr int kScaleMfmas = (NF + 1) / 2;              // MFMAs that carry two scale reads each
+        static_assert(kM == 16 && kB1 + kScaleMfmas + 1 <= 14, "the scale shift must sit at least two MFMAs before the end of the step");
         using SlotT = std::integral_constant<int, slot>;
         using OtherT = std::integral_constant<int, slot ^ 1>;
         const uint32_t k2 = clamp_slab(s + 2);
         const uint32_t koff = k2 * kSlabBytes, soff = k2 * 4;
         // ---- step 0 ----
-        static_for<0, 16>([&](auto ic) {
-            constexpr int i = decltype(ic)::value, fw = i / 4, fm = i % 4;
-            mfma_acc<FMT, 0>(acc[fw][fm], join8(f0lo[fw], f0hi[fw]), join8(f0lo[4 + fm], f0hi[4 + fm]), scur[slot][fw], scur[slot][4 + fm]);
-            if constexpr (i < 8) {
-                constexpr int idx = pipe_read_order(i);
-                if (!(CMX_PIPE_DBG & 4)) read_frag(SlotT{}, I1{}, std::integral_constant<int, idx>{}, f1lo[idx], f1hi[idx]);
-            }
+        static_for<0, kM>([&](auto ic) {
+            constexpr int i = decltype(ic)::value;
+            step_mfma(I0{}, ic, f0lo, f0hi, SlotT{});
+            static_for<0, kR>([&](auto jc) {
+                constexpr int r = i * kR + decltype(jc)::value;
+                if constexpr (r < kReads) read_half(SlotT{}, I1{}, std::integral_constant<int, r>{}, f1lo, f1hi);
+            });
             // slot `slot` has been read for the last time: once everyone is here it can be refilled
-            if constexpr (i == 16 - kEarly - 1) asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
-            if constexpr (i >= 16 - kEarly) {
-                if (!(CMX_PIPE_DBG & 1)) issue_tile_load(slot, i - (16 - kEarly), koff);
-            }
+            if constexpr (i == kB1) asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+            if constexpr (i > kB1) issue_tile_load(slot, i - kB1 - 1, koff);
         });
+        pin_fragments(f0lo, f0hi);
         // own loads of slab s+1 are complete (only the kEarly loads just issued may be in flight); after the
         // barrier so are everyone's
-        if (CMX_PIPE_DBG & 17) asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");
-        else asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(kEarly) : "memory");
+        asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(kEarly) : "memory");
         // ---- step 1 ----
-        static_for<0, 16>([&](auto ic) {
-            constexpr int i = decltype(ic)::value, fw = i / 4, fm = i % 4;
-            mfma_acc<FMT, 2>(acc[fw][fm], join8(f1lo[fw], f1hi[fw]), join8(f1lo[4 + fm], f1hi[4 + fm]), scur[slot][fw], scur[slot][4 + fm]);
-            if constexpr (i + kEarly < 16) {
-                if (!(CMX_PIPE_DBG & 1)) issue_tile_load(slot, i + kEarly, koff);
+        static_for<0, kM>([&](auto ic) {
+            constexpr int i = decltype(ic)::value;
+            step_mfma(I2{}, ic, f1lo, f1hi, SlotT{});
+            if constexpr (i + kEarly < kTileLoads) issue_tile_load(slot, i + kEarly, koff);
+            if constexpr (i + kEarly == kTileLoads) issue_scale_loads(slot, soff);
+            static_for<0, kR>([&](auto jc) {
+                constexpr int r = i * kR + decltype(jc)::value;
+                if constexpr (r < kReads) read_half(OtherT{}, I0{}, std::integral_constant<int, r>{}, f0lo, f0hi);
+            });
+            if constexpr (i >= kB1 && i < kB1 + kScaleMfmas) {
+                read_scale(OtherT{}, std::integral_constant<int, 2 * (i - kB1)>{});
+                if constexpr (2 * (i - kB1) + 1 < NF) read_scale(OtherT{}, std::integral_constant<int, 2 * (i - kB1) + 1>{});
             }
-            if constexpr (i + kEarly == 16) { if (!(CMX_PIPE_DBG & 8)) issue_scale_loads(slot, soff); }
-            if constexpr (i < 8) {
-                constexpr int idx = pipe_read_order(i);
-                if (!(CMX_PIPE_DBG & 4)) read_frag(OtherT{}, I0{}, std::integral_constant<int, idx>{}, f0lo[idx], f0hi[idx]);
-            } else if constexpr (i < 12) {
-                read_scale(OtherT{}, std::integral_constant<int, 2 * (i - 8)>{});
-                read_scale(OtherT{}, std::integral_constant<int, 2 * (i - 8) + 1>{});
-            }
-            if constexpr (i == 13) {
+            if constexpr (i == kB1 + kScaleMfmas + 1) {
                 asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
                 shift_scales(OtherT{});
             }
         });
-        // Keep this slab's scale registers allocated to the end of the slab: otherwise the shifts above may be
-        // given the register of a scale whose last reader is an MFMA issued a few cycles earlier, and nothing
-        // orders that VALU write behind the MFMA's operand fetch.
-#pragma unroll
-        for (int i = 0; i < 8; ++i) asm volatile("" ::"v"(scur[slot][i]));
+        pin_fragments(f1lo, f1hi);
+        pin_scales(SlotT{});
+    };
+
+    // ---- three-slot ring (8 MFMAs per step) -----------------------------------------------------------------
+    // While slab s (slot s%3) is consumed, slab s+1 is landing or landed and slab s+2 is in flight.  Half way
+    // through, everybody has read slot s%3 for the last time and waited for its own loads of slab s+1: one
+    // barrier frees the slot and publishes slab s+1, and the loads of slab s+3 go straight into the freed
+    // slot, so two slabs are in flight for two slab times each.
+    auto slab_body3 = [&](auto slot_c, uint32_t s) {
+        constexpr int slot = decltype(slot_c)::value;
+        static_assert(NSLOT == 2 || (kM == 8 && kReads == 12 && kTileLoads == 12 && NF == 6), "three-slot schedule is written for the 256 x 128 tile");
+        using SlotT = std::integral_constant<int, slot>;
+        using NextT = std::integral_constant<int, (slot + 1) % 3>;
+        const uint32_t k3 = clamp_slab(s + 3);
+        const uint32_t koff = k3 * kSlabBytes, soff = k3 * 4;
+        // ---- step 0: second half of the slab into fragment set 1 ----
+        static_for<0, kM>([&](auto ic) {
+            constexpr int i = decltype(ic)::value;
+            step_mfma(I0{}, ic, f0lo, f0hi, SlotT{});
+            if constexpr (2 * i < kReads) {
+                read_half(SlotT{}, I1{}, std::integral_constant<int, 2 * i>{}, f1lo, f1hi);
+                read_half(SlotT{}, I1{}, std::integral_constant<int, 2 * i + 1>{}, f1lo, f1hi);
+            }
+        });
+        pin_fragments(f0lo, f0hi);
+        // own reads of slot `slot` and own loads of slab s+1 are complete (slab s+2 may be in flight)
+        asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(kLoadsPerSlab) : "memory");
+        // ---- step 1: loads of slab s+3 into the freed slot, first half of slab s+1 into fragment set 0 ----
+        static_for<0, kM>([&](auto ic) {
+            constexpr int i = decltype(ic)::value;
+            step_mfma(I2{}, ic, f1lo, f1hi, SlotT{});
+            if constexpr (i < 3) {                 // the six scale dwords first: they are waited for before the fragments
+                read_scale(NextT{}, std::integral_constant<int, 2 * i>{});
+                read_scale(NextT{}, std::integral_constant<int, 2 * i + 1>{});
+            }
+            if constexpr (2 * i < kTileLoads) {
+                issue_tile_load(slot, 2 * i, koff);
+                issue_tile_load(slot, 2 * i + 1, koff);
+            }
+            if constexpr (2 * i == kTileLoads) issue_scale_loads(slot, soff);
+            if constexpr (2 * i < kReads) {
+                read_half(NextT{}, I0{}, std::integral_constant<int, 2 * i>{}, f0lo, f0hi);
+                read_half(NextT{}, I0{}, std::integral_constant<int, 2 * i + 1>{}, f0lo, f0hi);
+            }
+            if constexpr (i == 6) {
+                // LDS reads return in order, and 8 fragment reads (two of MFMA 2, all of MFMAs 3..5) were issued
+                // after the last scale read: the scales are in once at most those 8 are outstanding
+                asm volatile("s_waitcnt lgkmcnt(8)" ::: "memory");
+                shift_scales(NextT{});
+            }
+        });
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");      // fragment set 0 of the next slab
+        pin_fragments(f1lo, f1hi);
+        pin_scales(SlotT{});
     };
 
     // The compiler does not see the MFMAs inside the asm statements, so it inserts none of the wait states
     // that separate them from its own accumulator accesses.  Passing every accumulator through an asm
     // statement that holds the wait states pins those accesses to the far side of it.
     auto fence_accumulators = [&]() {
-        (void)acc;
-        asm volatile("s_nop 15\n\ts_nop 15"
-                     : "+a"(acc[0][0]), "+a"(acc[0][1]), "+a"(acc[0][2]), "+a"(acc[0][3]), "+a"(acc[1][0]), "+a"(acc[1][1]),
-                       "+a"(acc[1][2]), "+a"(acc[1][3]));
-        asm volatile("s_nop 15\n\ts_nop 15"
-                     : "+a"(acc[2][0]), "+a"(acc[2][1]), "+a"(acc[2][2]), "+a"(acc[2][3]), "+a"(acc[3][0]), "+a"(acc[3][1]),
-                       "+a"(acc[3][2]), "+a"(acc[3][3]));
+        v16f* const a = &acc[0][0];
+        asm volatile("s_nop 15\n\ts_nop 15" : "+a"(a[0]), "+a"(a[1]), "+a"(a[2]), "+a"(a[3]), "+a"(a[4]), "+a"(a[5]), "+a"(a[6]), "+a"(a[7]));
+        if constexpr (kM == 16)
+            asm volatile("s_nop 15\n\ts_nop 15" : "+a"(a[8]), "+a"(a[9]), "+a"(a[10]), "+a"(a[11]), "+a"(a[12]), "+a"(a[13]), "+a"(a[14]), "+a"(a[15]));
     };
     fence_accumulators();       // the zero initialisation has retired before the first MFMA reads it
-    for (uint32_t s = 0; s < nslab; s += 2) {      // the host only selects this kernel for an even slab count
-        slab_body(I0{}, s);
-        slab_body(I1{}, s + 1);
+    if constexpr (NSLOT == 2) {
+        for (uint32_t s = 0; s < nslab; s += 2) {      // the host only selects this kernel for an even slab count
+            slab_body2(I0{}, s);
+            slab_body2(I1{}, s + 1);
+        }
+    } else {
+        uint32_t s = 0;
+        for (; s + 3 <= nslab; s += 3) {
+            slab_body3(I0{}, s);
+            slab_body3(I1{}, s + 1);
+            slab_body3(I2{}, s + 2);
+        }
+        const uint32_t rem = nslab - s;                 // the ring position after whole turns is slot 0 again
+        if (rem >= 1) slab_body3(I0{}, s);
+        if (rem == 2) slab_body3(I1{}, s + 1);
     }
     // the loads issued past the end must land before the LDS is released; the last MFMAs must have
     // written their accumulators before the epilogue reads them

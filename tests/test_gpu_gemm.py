@@ -9,7 +9,7 @@ from tests.gpu_util import dev, host, close_bf16
 
 pytestmark = pytest.mark.gpu
 
-TILES = [(256, 256, 4), (256, 256, 8), (256, 128, 4), (256, 128, 8), (256, 64, 4), (128, 128, 4)]
+TILES = [(256, 256, 4), (256, 256, 5), (256, 128, 5), (256, 256, 8), (256, 128, 4), (256, 128, 8), (256, 64, 4), (128, 128, 4)]
 
 
 def _mx(rng, rows, k, fmt="E4M3", std=1.0):

@@ -22,7 +22,7 @@ def _weights(rng, g, n, k, std=0.05, fmt="E4M3"):
     return np.stack([q for q, _ in qs]), np.stack([s for _, s in qs])
 
 
-@pytest.mark.parametrize("tile", [None, (256, 256, 4), (256, 256, 8), (256, 128, 4), (256, 128, 8), (256, 64, 4), (128, 128, 4)])
+@pytest.mark.parametrize("tile", [None, (256, 256, 4), (256, 256, 5), (256, 128, 5), (256, 256, 8), (256, 128, 4), (256, 128, 8), (256, 64, 4), (128, 128, 4)])
 @pytest.mark.parametrize("counts", [[5, 0, 300, 1, 0, 257, 64], [0, 0, 7], [512], [1] * 9])
 def test_gmm_fp8_ragged_groups(tile, counts):
     from catccos_amd import ops, _lib
@@ -57,7 +57,7 @@ def test_gmm_fp4_ragged_groups():
     assert np.allclose(host(c).astype(np.float64), gold, rtol=2e-3, atol=5e-2)
 
 
-@pytest.mark.parametrize("tile", [None, (256, 256, 4), (256, 256, 8), (256, 128, 4), (256, 128, 8), (256, 64, 4), (128, 128, 4)])
+@pytest.mark.parametrize("tile", [None, (256, 256, 4), (256, 256, 5), (256, 128, 5), (256, 256, 8), (256, 128, 4), (256, 128, 8), (256, 64, 4), (128, 128, 4)])
 def test_gmm1_swiglu_requant(tile):
     """h and act are within tolerance of the golden chain; the requantised codes and scales are
     bit-exact against the oracle quantizer applied to the kernel's own bf16 SwiGLU output."""
