@@ -136,6 +136,39 @@ __device__ __forceinline__ uint32_t e2m1_encode(float y, bool lut) {
     return c | ((__float_as_uint(y) >> 28) & 8u);
 }
 
+
+// ---- packed 16-bit helpers (bf16 bit patterns) and the scaled hardware casts of gfx950 ----------------
+typedef unsigned short v2u16 __attribute__((ext_vector_type(2)));
+typedef short v2i16 __attribute__((ext_vector_type(2)));
+typedef __bf16 v2bf16 __attribute__((ext_vector_type(2)));
+
+__device__ __forceinline__ uint32_t pk_max_u16(uint32_t a, uint32_t b) {
+    return __builtin_bit_cast(uint32_t, __builtin_elementwise_max(__builtin_bit_cast(v2u16, a), __builtin_bit_cast(v2u16, b)));
+}
+__device__ __forceinline__ uint32_t pk_min_u16(uint32_t a, uint32_t b) {
+    return __builtin_bit_cast(uint32_t, __builtin_elementwise_min(__builtin_bit_cast(v2u16, a), __builtin_bit_cast(v2u16, b)));
+}
+
+template <int FMT>
+__device__ __forceinline__ uint32_t cvt_scaled_pk4(uint32_t d0, uint32_t d1, float scale) {
+    v2i16 o = {0, 0};
+    if constexpr (FMT == CMX_FMT_E4M3) {
+        o = __builtin_amdgcn_cvt_scalef32_pk_fp8_bf16(o, __builtin_bit_cast(v2bf16, d0), scale, false);
+        o = __builtin_amdgcn_cvt_scalef32_pk_fp8_bf16(o, __builtin_bit_cast(v2bf16, d1), scale, true);
+    } else {
+        o = __builtin_amdgcn_cvt_scalef32_pk_bf8_bf16(o, __builtin_bit_cast(v2bf16, d0), scale, false);
+        o = __builtin_amdgcn_cvt_scalef32_pk_bf8_bf16(o, __builtin_bit_cast(v2bf16, d1), scale, true);
+    }
+    return __builtin_bit_cast(uint32_t, o);
+}
+
+
+typedef float v2f32 __attribute__((ext_vector_type(2)));
+// two floats -> packed bf16 (a in the low half), round-to-nearest-even in hardware
+__device__ __forceinline__ uint32_t cvt_pk_bf16(float a, float b) {
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector((v2f32){a, b}, v2bf16));
+}
+
 #endif  // __HIPCC__
 
 }  // namespace cmx

@@ -45,6 +45,7 @@ struct GemmParams {
     uint16_t* act_bf16;
     const int32_t* row_off;     // [groups+1] (grouped) or null (dense)
     const int32_t* tile_pref;   // [groups+1] prefix of m-tiles (grouped) or null
+    int32_t* tile_ctr;          // [8] per-XCD tile counters, zeroed before the launch (persistent grouped kernels) or null
     uint32_t lda, ld_as, ldw, ld_ws, ldc, ld_act, ld_acts;
     uint32_t m, n, kbytes, kblocks;   // kblocks = K/32
     uint32_t groups, w_tiles;
@@ -96,8 +97,10 @@ __device__ __forceinline__ v16f mfma<CMX_FMT_E2M1>(v8i w, v8i a, v16f c, int sel
     }
 }
 
+// g / (1 + exp(-g)) * u with the hardware exponential and reciprocal (about 1 ulp each; the result is rounded
+// to bf16 right after)
 __device__ __forceinline__ float silu_mul(float g, float u) {
-    float s = 1.0f / (1.0f + __expf(-g));
+    const float s = __builtin_amdgcn_rcpf(1.0f + __expf(-g));
     return (g * s) * u;
 }
 
@@ -105,19 +108,24 @@ struct Tile {
     uint32_t g, mt, wt, row0, rows_valid;
 };
 
-// Maps the workgroup id to (group, m-tile, weight tile).  Returns false for ids past the last tile.
+// Tiles are numbered linearly: within a group m-tiles run fastest so that neighbours share a weight panel;
+// dense problems walk bands of four m-tiles across a run of weight tiles.
 template <int TM>
-__device__ __forceinline__ bool locate_tile(const GemmParams& p, Tile& t) {
-    const uint32_t grouped = p.row_off != nullptr;
-    const uint32_t m_tiles_all = grouped ? (uint32_t)p.tile_pref[p.groups] : (p.m + TM - 1) / TM;
-    const uint32_t total_tiles = m_tiles_all * p.w_tiles;
-    const uint32_t bid = blockIdx.x;
-    if (bid >= total_tiles) return false;
-    // XCD-aware remap: ids congruent mod 8 run on one XCD; give each a contiguous run of tiles.
-    const uint32_t x = bid % kXcds, j = bid / kXcds;
+__device__ __forceinline__ uint32_t count_m_tiles(const GemmParams& p) {
+    return p.row_off != nullptr ? (uint32_t)p.tile_pref[p.groups] : (p.m + TM - 1) / TM;
+}
+
+// Tile L of an XCD-aware order: linear ids congruent mod 8 run on one XCD; each XCD gets a contiguous run.
+// Returns the first tile of XCD x and the number of tiles it owns.
+__device__ __forceinline__ uint32_t xcd_run(uint32_t total_tiles, uint32_t x, uint32_t& count) {
     const uint32_t base = total_tiles / kXcds, rem = total_tiles % kXcds;
-    const uint32_t L = x * base + (x < rem ? x : rem) + j;
-    if (grouped) {
+    count = base + (x < rem ? 1u : 0u);
+    return x * base + (x < rem ? x : rem);
+}
+
+template <int TM>
+__device__ __forceinline__ void decode_tile(const GemmParams& p, uint32_t m_tiles_all, uint32_t L, Tile& t) {
+    if (p.row_off != nullptr) {
         // find g with tile_pref[g]*w_tiles <= L < tile_pref[g+1]*w_tiles
         uint32_t lo = 0, hi = p.groups;
         while (hi - lo > 1) {
@@ -145,6 +153,19 @@ __device__ __forceinline__ bool locate_tile(const GemmParams& p, Tile& t) {
         t.row0 = t.mt * TM;
         t.rows_valid = p.m - t.row0 < (uint32_t)TM ? p.m - t.row0 : (uint32_t)TM;
     }
+}
+
+// One tile per workgroup: maps the workgroup id to (group, m-tile, weight tile).  Returns false for ids past
+// the last tile.
+template <int TM>
+__device__ __forceinline__ bool locate_tile(const GemmParams& p, Tile& t) {
+    const uint32_t m_tiles_all = count_m_tiles<TM>(p);
+    const uint32_t total_tiles = m_tiles_all * p.w_tiles;
+    const uint32_t bid = blockIdx.x;
+    if (bid >= total_tiles) return false;
+    uint32_t count;
+    const uint32_t L = xcd_run(total_tiles, bid % kXcds, count) + bid / kXcds;
+    decode_tile<TM>(p, m_tiles_all, L, t);
     return true;
 }
 
@@ -207,34 +228,40 @@ __device__ __forceinline__ void epilogue(const GemmParams& p, const Tile& tc, v1
             for (int f = 0; f < FW / 2; ++f) {
                 // activation column of this fragment's 32-wide MX block
                 const uint32_t ncol0 = wt * (TW / 2) + ww * (TW / 2 / WW) + f * 32;
-                float actv[16];
-                uint32_t amax = 0;
+                // GMM1 output rounded to bf16, SwiGLU in fp32, rounded to bf16 again: all on packed pairs with the
+                // hardware bf16 conversion; pk[j] holds activation values 2j, 2j+1 of this lane
+                uint32_t pk[8];
+                uint32_t m = 0;
 #pragma unroll
-                for (int r = 0; r < 16; ++r) {
-                    const float hg = bf16_to_f32(f32_to_bf16(acc[f][fm][r]));
-                    const float hu = bf16_to_f32(f32_to_bf16(acc[f + FW / 2][fm][r]));
-                    const uint32_t ab = f32_to_bf16(silu_mul(hg, hu));
-                    actv[r] = bf16_to_f32(ab);
-                    const uint32_t mag = ab & 0x7FFFu;
-                    amax = amax > mag ? amax : mag;
-                    if (p.act_bf16 && mvalid) {
+                for (int j = 0; j < 8; ++j) {
+                    const uint32_t g2 = cvt_pk_bf16(acc[f][fm][2 * j], acc[f][fm][2 * j + 1]);
+                    const uint32_t u2 = cvt_pk_bf16(acc[f + FW / 2][fm][2 * j], acc[f + FW / 2][fm][2 * j + 1]);
+                    const float a0 = silu_mul(__uint_as_float(g2 << 16), __uint_as_float(u2 << 16));
+                    const float a1 = silu_mul(__uint_as_float(g2 & 0xFFFF0000u), __uint_as_float(u2 & 0xFFFF0000u));
+                    pk[j] = cvt_pk_bf16(a0, a1);
+                    m = pk_max_u16(m, pk[j] & 0x7FFF7FFFu);
+                }
+                if (p.act_bf16 && mvalid) {
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) {
                         const uint32_t ncol = ncol0 + 8 * (r >> 2) + 4 * lh + (r & 3);
-                        if (ncol < half) p.act_bf16[mrow * half + ncol] = (uint16_t)ab;
+                        if (ncol < half) p.act_bf16[mrow * half + ncol] = (uint16_t)(pk[r >> 1] >> (16 * (r & 1)));
                     }
                 }
+                uint32_t amax = max(m & 0xFFFFu, m >> 16);
                 const uint32_t other = (uint32_t)__shfl_xor((int)amax, 32);
                 amax = amax > other ? amax : other;
                 const int e = block_exp_from_bf16_amax(amax, kEmaxE4M3);
                 if (!mvalid || ncol0 >= half) continue;
+                // clamp the magnitudes to 448 * 2^e on the bit patterns, divide by 2^e and cast in one instruction
+                const uint32_t lim = (((uint32_t)(e + kEmaxE4M3 + 127) << 7) | 0x60u) * 0x10001u;
+                const float scale = __uint_as_float((uint32_t)(e + 127) << 23);
 #pragma unroll
                 for (int q = 0; q < 4; ++q) {
-                    float y0 = clamp_abs(ldexpf(actv[4 * q + 0], -e), 448.0f);
-                    float y1 = clamp_abs(ldexpf(actv[4 * q + 1], -e), 448.0f);
-                    float y2 = clamp_abs(ldexpf(actv[4 * q + 2], -e), 448.0f);
-                    float y3 = clamp_abs(ldexpf(actv[4 * q + 3], -e), 448.0f);
-                    uint32_t wv = cvt_pk_e4m3(y0, y1, 0u, false);
-                    wv = cvt_pk_e4m3(y2, y3, wv, true);
-                    *reinterpret_cast<uint32_t*>(p.act_codes + mrow * p.ld_act + ncol0 + 8 * q + 4 * lh) = wv;
+                    const uint32_t c0 = pk_min_u16(pk[2 * q] & 0x7FFF7FFFu, lim) | (pk[2 * q] & 0x80008000u);
+                    const uint32_t c1 = pk_min_u16(pk[2 * q + 1] & 0x7FFF7FFFu, lim) | (pk[2 * q + 1] & 0x80008000u);
+                    *reinterpret_cast<uint32_t*>(p.act_codes + mrow * p.ld_act + ncol0 + 8 * q + 4 * lh) =
+                        cvt_scaled_pk4<CMX_FMT_E4M3>(c0, c1, scale);
                 }
                 if (lh == 0) {
                     uint8_t* srow = p.act_scales + mrow * p.ld_acts;
@@ -702,8 +729,10 @@ __global__ __launch_bounds__(64 * WW * WM) void mx_gemm_dl_kernel(const GemmPara
 
 // Row offsets and m-tile prefix of the groups (one workgroup).
 __global__ void gmm_prepare_kernel(const int32_t* __restrict__ sizes, uint32_t groups, uint32_t tile_m,
-                                   int32_t* __restrict__ row_off, int32_t* __restrict__ tile_pref) {
+                                   int32_t* __restrict__ row_off, int32_t* __restrict__ tile_pref,
+                                   int32_t* __restrict__ tile_ctr) {
     extern __shared__ int32_t sh[];
+    if (threadIdx.x < kXcds) tile_ctr[threadIdx.x] = 0;
     for (uint32_t i = threadIdx.x; i < groups; i += blockDim.x) sh[i] = sizes[i] > 0 ? sizes[i] : 0;
     __syncthreads();
     if (threadIdx.x == 0) {
@@ -757,7 +786,7 @@ int launch_gemm_dl(const GemmParams& p, uint32_t max_m_tiles, hipStream_t s) {
 
 template <int FMT, int EPI, int TM, int WW, int WM, int NSLOT>
 int launch_gemm_pipe(const GemmParams& p, uint32_t max_m_tiles, hipStream_t s) {
-    constexpr size_t smem = NSLOT * (256 + TM) * (kSlabBytes + 4);
+    constexpr size_t smem = NSLOT * (256 + TM) * (kSlabBytes + 4) + 16;     // ring, scale ring, next-tile mailbox
     auto kfn = mx_gemm_pipe_kernel<FMT, EPI, TM, WW, WM, NSLOT>;
     static bool attr_set = false;
     if (!attr_set) {
@@ -767,7 +796,20 @@ int launch_gemm_pipe(const GemmParams& p, uint32_t max_m_tiles, hipStream_t s) {
     }
     const uint64_t tiles = (uint64_t)max_m_tiles * p.w_tiles;
     CMX_REQUIRE(tiles > 0 && tiles < (1ull << 31), "tile count out of range");
-    hipLaunchKernelGGL(kfn, dim3((uint32_t)tiles), dim3(256), smem, s, p);
+    uint32_t grid = (uint32_t)tiles;
+    if (pipe_is_persistent(NSLOT, EPI)) {
+        // persistent: one workgroup per CU (the LDS footprint admits no second one), a multiple of the XCD count
+        static int cus = 0;
+        if (cus == 0) {
+            int dev = 0, n = 0;
+            CMX_HIP(hipGetDevice(&dev));
+            CMX_HIP(hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev));
+            cus = n > 0 ? n : 256;
+        }
+        grid = (uint32_t)(cus / kXcds * kXcds);
+        if (grid < (uint32_t)kXcds) grid = kXcds;
+    }
+    hipLaunchKernelGGL(kfn, dim3(grid), dim3(256), smem, s, p);
     CMX_LAUNCH_CHECK();
     return CMX_OK;
 }
@@ -894,7 +936,8 @@ extern "C" int cmx_mx_gemm(const uint8_t* a, uint32_t lda, const uint8_t* a_scal
 }
 
 extern "C" size_t cmx_mx_gmm_workspace_bytes(uint32_t groups) {
-    return cmx::round_up_sz(2 * (size_t)(groups + 1) * sizeof(int32_t), 256);
+    // row offsets, m-tile prefix, per-XCD tile counters
+    return cmx::round_up_sz((2 * (size_t)(groups + 1) + 8) * sizeof(int32_t), 256);
 }
 
 namespace cmx {
@@ -910,11 +953,13 @@ int gmm_common(GemmParams& p, const int32_t* group_sizes, uint32_t groups, uint3
     TileChoice t = choose_tile(ceil_div(m_total, groups), p.n, fmt, true);
     int32_t* row_off = static_cast<int32_t*>(workspace);
     int32_t* tile_pref = row_off + (groups + 1);
+    int32_t* tile_ctr = tile_pref + (groups + 1);
     hipLaunchKernelGGL(gmm_prepare_kernel, dim3(1), dim3(256), groups * sizeof(int32_t), s, group_sizes, groups,
-                       (uint32_t)t.tm, row_off, tile_pref);
+                       (uint32_t)t.tm, row_off, tile_pref, tile_ctr);
     CMX_LAUNCH_CHECK();
     p.row_off = row_off;
     p.tile_pref = tile_pref;
+    p.tile_ctr = tile_ctr;
     p.groups = groups;
     p.w_tiles = swiglu ? ceil_div(p.n / 2, t.tw / 2) : ceil_div(p.n, t.tw);
     const uint32_t max_m_tiles = m_total / t.tm + groups;

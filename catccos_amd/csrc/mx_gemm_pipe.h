@@ -77,6 +77,7 @@ __device__ __forceinline__ void dma_b32(uint32_t lds_dst, uint32_t voff, v4i rsr
 template <int FMT, int SEL, int BIT>
 __device__ __forceinline__ void mfma_acc(v16f& acc, const v8i& w, const v8i& a, uint32_t sw, uint32_t sa, uint32_t live) {
     static_assert(SEL == 0 || SEL == 2, "scale byte pair");
+    live = __builtin_amdgcn_readfirstlane(live);      // uniform by construction; makes it a scalar operand for certain
     if constexpr (FMT == CMX_FMT_E4M3) {
         if constexpr (SEL == 0) { CMX_PIPE_MFMA("[0,0,0]", ""); } else { CMX_PIPE_MFMA("[1,1,0]", ""); }
     } else {
@@ -106,6 +107,8 @@ __device__ __forceinline__ v8i join8(const v4i& lo, const v4i& hi) {
 //   TM 128, 3 slots, 4 x 1: two slabs instead of one in flight behind the one being consumed, for groups
 //           so short that every tile streams its weights from HBM once and the load latency, not the MFMA
 //           rate, sets the pace.
+__host__ __device__ constexpr bool pipe_is_persistent(int nslot, int epi) { return nslot == 2 && epi == kEpiSwigluQuant; }
+
 template <int FMT, int EPI, int TM, int WW, int WM, int NSLOT>
 __global__ __launch_bounds__(256) void mx_gemm_pipe_kernel(const GemmParams p) {
     static_assert(FMT == CMX_FMT_E4M3 || FMT == CMX_FMT_E5M2, "8-bit element formats only");
@@ -132,49 +135,26 @@ __global__ __launch_bounds__(256) void mx_gemm_pipe_kernel(const GemmParams p) {
     const uint32_t ww = wave % WW, wm = wave / WW;
     const uint32_t l32 = lane & 31u, lh = lane >> 5;
 
-    Tile tc;
-    if (!locate_tile<TM>(p, tc)) return;
-    const uint32_t g = __builtin_amdgcn_readfirstlane(tc.g), wt = __builtin_amdgcn_readfirstlane(tc.wt);
-    const uint32_t row0 = __builtin_amdgcn_readfirstlane(tc.row0);
-    const uint32_t rows_valid = __builtin_amdgcn_readfirstlane(tc.rows_valid);
+    // ---- tile sequence of this workgroup ------------------------------------------------------------------
+    // The two-slot kernels with the SwiGLU epilogue are persistent: the grid is one workgroup per CU, and
+    // workgroup j of XCD x walks tiles j, j + (workgroups per XCD), ... of that XCD's contiguous run, carrying
+    // the load pipeline across tile boundaries.  The others take one tile per workgroup (the plain store
+    // epilogue with its three output types and edge cases needs too many registers to sit inside the loop).
+    constexpr bool kPersistent = pipe_is_persistent(NSLOT, EPI);
+    const uint32_t m_tiles_all = count_m_tiles<TM>(p);
+    const uint32_t total_tiles = m_tiles_all * p.w_tiles;
+    uint32_t run_count;
+    const uint32_t run_first = xcd_run(total_tiles, blockIdx.x % kXcds, run_count);
+    const uint32_t run_end = run_first + run_count;
+    const uint32_t tile_stride = kPersistent ? gridDim.x / kXcds : total_tiles;      // one tile only when not persistent
+    uint32_t tile_id = run_first + blockIdx.x / kXcds;
+    if (tile_id >= run_end) return;
 
-    const uint8_t* wg = p.w + (size_t)g * p.n * p.ldw;
-    const uint8_t* wsg = p.w_scale + (size_t)g * p.n * p.ld_ws;
-    const uint8_t* ag = p.a + (size_t)row0 * p.lda;
-    const uint8_t* asg = p.a_scale + (size_t)row0 * p.ld_as;
-
-    // global row of tile row r (rows past the edge re-read the last valid row; their results are never stored)
-    auto wrow_of = [&](uint32_t r) -> uint32_t {
-        uint32_t gr;
-        if (EPI == kEpiSwigluQuant) {
-            const uint32_t half = p.n >> 1;
-            uint32_t rr = r < TW / 2 ? wt * (TW / 2) + r : wt * (TW / 2) + (r - TW / 2);
-            rr = rr < half ? rr : half - 1;
-            gr = r < TW / 2 ? rr : half + rr;
-        } else {
-            gr = wt * TW + r;
-            gr = gr < p.n ? gr : p.n - 1;
-        }
-        return gr;
-    };
-    auto arow_of = [&](uint32_t r) -> uint32_t { return r < rows_valid ? r : rows_valid - 1; };
-
-    // ---- LDS-DMA: per-lane global offsets (constant over K) ---------------------------------------
-    // load i of this wavefront fills combined tile rows (4i + wave)*8 .. +8; lane q -> row +q/8, LDS
-    // chunk q%8, and fetches the global chunk that the XOR swizzle maps there
-    uint32_t goff[kTileLoads];
-#pragma unroll
-    for (int i = 0; i < kTileLoads; ++i) {
-        const uint32_t cr = (NW * i + wave) * 8 + (lane >> 3);
-        const uint32_t logical = swz(cr, lane & 7u);
-        goff[i] = (i < kWTileLoads ? wrow_of(cr) * p.ldw : arow_of(cr - TW) * p.lda) + logical * 16;
-    }
-    // scale dwords: this wavefront fetches those of weight rows 64*wave.. and of activation rows 64*(wave mod TM/64)..
-    // (with TM = 128 two wavefronts fetch the same rows to the same place)
+    // addressing of the tile whose slabs are being requested (switches two slabs before a tile boundary)
+    Tile tq;                                    // tile of the load stream
+    v4i w_rs, a_rs, ws_rs, as_rs;
+    uint32_t goff[kTileLoads], sgoff_w, sgoff_a;
     const uint32_t sa_blk = wave % (TM / 64);
-    const uint32_t sgoff_w = wrow_of(64 * wave + lane) * p.ld_ws;
-    const uint32_t sgoff_a = arow_of(64 * sa_blk + lane) * p.ld_as;
-
     auto make_rsrc = [](const uint8_t* q) -> v4i {
         const uint64_t v = reinterpret_cast<uint64_t>(q);
         v4i r;
@@ -184,7 +164,47 @@ __global__ __launch_bounds__(256) void mx_gemm_pipe_kernel(const GemmParams p) {
         r[3] = 0x00020000;
         return r;
     };
-    const v4i w_rs = make_rsrc(wg), a_rs = make_rsrc(ag), ws_rs = make_rsrc(wsg), as_rs = make_rsrc(asg);
+    auto aim_loads_at = [&](uint32_t L) {
+        decode_tile<TM>(p, m_tiles_all, L, tq);
+        const uint32_t g = __builtin_amdgcn_readfirstlane(tq.g), wt = __builtin_amdgcn_readfirstlane(tq.wt);
+        const uint32_t row0 = __builtin_amdgcn_readfirstlane(tq.row0);
+        const uint32_t rows_valid = __builtin_amdgcn_readfirstlane(tq.rows_valid);
+        tq.g = g; tq.wt = wt; tq.row0 = row0; tq.rows_valid = rows_valid;
+        tq.mt = __builtin_amdgcn_readfirstlane(tq.mt);
+        w_rs = make_rsrc(p.w + (size_t)g * p.n * p.ldw);
+        ws_rs = make_rsrc(p.w_scale + (size_t)g * p.n * p.ld_ws);
+        a_rs = make_rsrc(p.a + (size_t)row0 * p.lda);
+        as_rs = make_rsrc(p.a_scale + (size_t)row0 * p.ld_as);
+        // global row of tile row r (rows past the edge re-read the last valid row; their results are never stored)
+        auto wrow_of = [&](uint32_t r) -> uint32_t {
+            uint32_t gr;
+            if (EPI == kEpiSwigluQuant) {
+                const uint32_t half = p.n >> 1;
+                uint32_t rr = r < TW / 2 ? wt * (TW / 2) + r : wt * (TW / 2) + (r - TW / 2);
+                rr = rr < half ? rr : half - 1;
+                gr = r < TW / 2 ? rr : half + rr;
+            } else {
+                gr = wt * TW + r;
+                gr = gr < p.n ? gr : p.n - 1;
+            }
+            return gr;
+        };
+        auto arow_of = [&](uint32_t r) -> uint32_t { return r < rows_valid ? r : rows_valid - 1; };
+        // LDS-DMA load i of this wavefront fills combined tile rows (4i + wave)*8 .. +8; lane q -> row +q/8, LDS
+        // chunk q%8, and fetches the global chunk that the XOR swizzle maps there
+#pragma unroll
+        for (int i = 0; i < kTileLoads; ++i) {
+            const uint32_t cr = (NW * i + wave) * 8 + (lane >> 3);
+            const uint32_t logical = swz(cr, lane & 7u);
+            goff[i] = (i < kWTileLoads ? wrow_of(cr) * p.ldw : arow_of(cr - TW) * p.lda) + logical * 16;
+        }
+        // scale dwords: this wavefront fetches those of weight rows 64*wave.. and of activation rows
+        // 64*(wave mod TM/64).. (with TM = 128 two wavefronts fetch the same rows to the same place)
+        sgoff_w = wrow_of(64 * wave + lane) * p.ld_ws;
+        sgoff_a = arow_of(64 * sa_blk + lane) * p.ld_as;
+    };
+    aim_loads_at(tile_id);
+    Tile tc = tq;                               // tile of the MFMA stream / epilogue
 
     const uint32_t nslab = p.kbytes / kSlabBytes;
     const uint32_t dma_base = __builtin_amdgcn_readfirstlane(lds0 + wave * 1024);
@@ -283,7 +303,8 @@ __global__ __launch_bounds__(256) void mx_gemm_pipe_kernel(const GemmParams p) {
     shift_scales(I0{});
 
     // activation blocks of 32 rows that hold valid rows (4 x 1 layout: the others are skipped)
-    const uint32_t live = __builtin_amdgcn_readfirstlane((1u << ((rows_valid + 31) / 32)) - 1u);   // bit fm: block has valid rows
+    auto live_mask = [](uint32_t rows_valid) -> uint32_t { return __builtin_amdgcn_readfirstlane((1u << ((rows_valid + 31) / 32)) - 1u); };
+    uint32_t live = live_mask(tc.rows_valid);      // bit fm: block fm has valid rows
     auto step_mfma = [&](auto sel_c, auto i_c, v4i (&flo)[NF], v4i (&fhi)[NF], auto set_c) {
         constexpr int sel = decltype(sel_c)::value, i = decltype(i_c)::value, set = decltype(set_c)::value;
         constexpr int fw = kMOuter ? i % FW : i / FM, fm = kMOuter ? i / FW : i % FM;
@@ -313,7 +334,7 @@ __global__ __launch_bounds__(256) void mx_gemm_pipe_kernel(const GemmParams p) {
     // fragment set 0 and the shifted scales of the slab are in registers.  kR reads go behind each of the first
     // MFMAs of a step; after MFMA kB1 the last of them has had time to land; kEarly tile loads of slab s+2
     // are issued already in step 0, behind the first barrier.
-    auto slab_body2 = [&](auto slot_c, uint32_t s) {
+    auto slab_body2 = [&](auto slot_c, uint32_t koff, uint32_t soff) {
         constexpr int slot = decltype(slot_c)::value;
         constexpr int kR = NF > 8 ? 3 : 2;
         constexpr int kB1 = (kReads + kR - 1) / kR;
@@ -322,8 +343,6 @@ __global__ __launch_bounds__(256) void mx_gemm_pipe_kernel(const GemmParams p) {
         static_assert(kM == 16 && kB1 + kScaleMfmas + 1 <= 14, "the scale shift must sit at least two MFMAs before the end of the step");
         using SlotT = std::integral_constant<int, slot>;
         using OtherT = std::integral_constant<int, slot ^ 1>;
-        const uint32_t k2 = clamp_slab(s + 2);
-        const uint32_t koff = k2 * kSlabBytes, soff = k2 * 4;
         // ---- step 0 ----
         static_for<0, kM>([&](auto ic) {
             constexpr int i = decltype(ic)::value;
@@ -426,12 +445,7 @@ __global__ __launch_bounds__(256) void mx_gemm_pipe_kernel(const GemmParams p) {
             asm volatile("s_nop 15\n\ts_nop 15" : "+a"(a[8]), "+a"(a[9]), "+a"(a[10]), "+a"(a[11]), "+a"(a[12]), "+a"(a[13]), "+a"(a[14]), "+a"(a[15]));
     };
     fence_accumulators();       // the zero initialisation has retired before the first MFMA reads it
-    if constexpr (NSLOT == 2) {
-        for (uint32_t s = 0; s < nslab; s += 2) {      // the host only selects this kernel for an even slab count
-            slab_body2(I0{}, s);
-            slab_body2(I1{}, s + 1);
-        }
-    } else {
+    if constexpr (NSLOT == 3) {
         uint32_t s = 0;
         for (; s + 3 <= nslab; s += 3) {
             slab_body3(I0{}, s);
@@ -441,12 +455,78 @@ __global__ __launch_bounds__(256) void mx_gemm_pipe_kernel(const GemmParams p) {
         const uint32_t rem = nslab - s;                 // the ring position after whole turns is slot 0 again
         if (rem >= 1) slab_body3(I0{}, s);
         if (rem == 2) slab_body3(I1{}, s + 1);
+        // the loads issued past the end must land before the LDS is released; the last MFMAs must have
+        // written their accumulators before the epilogue reads them
+        asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+        fence_accumulators();
+        epilogue<TW, TM, WW, WM, EPI, FW, FM>(p, tc, acc, ww, wm, lane);
+    } else if constexpr (!kPersistent) {
+        for (uint32_t s = 0; s < nslab; s += 2) {      // the host only selects this kernel for an even slab count
+            const uint32_t q0 = clamp_slab(s + 2), q1 = clamp_slab(s + 3);
+            slab_body2(I0{}, q0 * kSlabBytes, q0 * 4);
+            slab_body2(I1{}, q1 * kSlabBytes, q1 * 4);
+        }
+        asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+        fence_accumulators();
+        epilogue<TW, TM, WW, WM, EPI, FW, FM>(p, tc, acc, ww, wm, lane);
+    } else {
+        // The host only selects this kernel for an even slab count.  The load stream runs two slabs ahead of
+        // the MFMA stream: when it reaches the end of the tile it is aimed at the workgroup's next tile (or keeps
+        // re-requesting the last slab when there is none), so the loads and the fragment reads run on through
+        // the tile boundary and only the epilogue and the clearing of the accumulators interrupt the MFMAs.
+        // One loop holds every case so that the register assignment of the scheduled part never changes.
+        // Next tile: with a counter array (grouped problems, whose tiles differ in cost) the workgroups of an
+        // XCD draw from that XCD's run in order; without one the walk is strided.
+        uint32_t sm = 0;             // slab of the MFMA stream within its tile
+        uint32_t sq = 2;             // slab of the load stream within its tile
+        bool next_ok = false;        // the load stream has moved on to a next tile
+        uint32_t next_id = tile_id;
+        for (;;) {
+            if (sq == nslab) {
+                if (p.tile_ctr != nullptr) {
+                    uint32_t* const mailbox = reinterpret_cast<uint32_t*>(smem + kScaleBase + NSLOT * kScaleSlotBytes);
+                    if (tid == 0) *mailbox = atomicAdd(reinterpret_cast<unsigned int*>(p.tile_ctr) + blockIdx.x % kXcds, 1u);
+                    __syncthreads();
+                    next_id = run_first + tile_stride + __builtin_amdgcn_readfirstlane(*mailbox);
+                } else {
+                    next_id = tile_id + tile_stride;
+                }
+                next_ok = next_id < run_end;
+                if (next_ok) {
+                    aim_loads_at(next_id);
+                    sq = 0;
+                }
+            }
+            const uint32_t q0 = clamp_slab(sq), q1 = clamp_slab(sq + 1);
+            slab_body2(I0{}, q0 * kSlabBytes, q0 * 4);
+            slab_body2(I1{}, q1 * kSlabBytes, q1 * 4);
+            sq += 2;
+            sm += 2;
+            if (sm == nslab) {
+                fence_accumulators();           // the last MFMAs have written their accumulators
+                epilogue<TW, TM, WW, WM, EPI, FW, FM>(p, tc, acc, ww, wm, lane);
+                if (!next_ok) break;
+                tile_id = next_id;
+                tc = tq;
+                live = live_mask(tc.rows_valid);
+                next_ok = false;
+                sm = 0;
+#pragma unroll
+                for (int i = 0; i < FW; ++i)
+#pragma unroll
+                    for (int j = 0; j < FM; ++j)
+#pragma unroll
+                        for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+                fence_accumulators();
+                // The last slab has already read the new tile's first fragments and scales, but carrying them
+                // through the epilogue costs more registers than there are: read them again (slot 0, landed).
+                static_for<0, NF>([&](auto ic) { read_frag(I0{}, I0{}, ic, f0lo, f0hi); });
+                static_for<0, NF>([&](auto ic) { read_scale(I0{}, ic); });
+                asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+                shift_scales(I0{});
+            }
+        }
+        asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");     // the re-requested slabs land before the LDS is released
     }
-    // the loads issued past the end must land before the LDS is released; the last MFMAs must have
-    // written their accumulators before the epilogue reads them
-    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
-    fence_accumulators();
 #undef CMX_PIPE_WOFF
-
-    epilogue<TW, TM, WW, WM, EPI, FW, FM>(p, tc, acc, ww, wm, lane);
 }

@@ -147,31 +147,7 @@ __global__ __launch_bounds__(kThreads) void mx_quant_kernel(const uint16_t* __re
 // +-max_normal * 2^e work on sign-cleared bf16 bit patterns (unsigned order == magnitude order), and
 // v_cvt_scalef32_pk_{fp8,bf8}_bf16 divides by 2^e and rounds to nearest even in one instruction.
 // Each lane of a quad then stores the scale byte of one of the four rows.
-typedef unsigned short v2u16 __attribute__((ext_vector_type(2)));
-typedef short v2i16 __attribute__((ext_vector_type(2)));
-typedef __bf16 v2bf16 __attribute__((ext_vector_type(2)));
-
 constexpr int kFastRows = 4;
-
-__device__ __forceinline__ uint32_t pk_max_u16(uint32_t a, uint32_t b) {
-    return __builtin_bit_cast(uint32_t, __builtin_elementwise_max(__builtin_bit_cast(v2u16, a), __builtin_bit_cast(v2u16, b)));
-}
-__device__ __forceinline__ uint32_t pk_min_u16(uint32_t a, uint32_t b) {
-    return __builtin_bit_cast(uint32_t, __builtin_elementwise_min(__builtin_bit_cast(v2u16, a), __builtin_bit_cast(v2u16, b)));
-}
-
-template <int FMT>
-__device__ __forceinline__ uint32_t cvt_scaled_pk4(uint32_t d0, uint32_t d1, float scale) {
-    v2i16 o = {0, 0};
-    if constexpr (FMT == CMX_FMT_E4M3) {
-        o = __builtin_amdgcn_cvt_scalef32_pk_fp8_bf16(o, __builtin_bit_cast(v2bf16, d0), scale, false);
-        o = __builtin_amdgcn_cvt_scalef32_pk_fp8_bf16(o, __builtin_bit_cast(v2bf16, d1), scale, true);
-    } else {
-        o = __builtin_amdgcn_cvt_scalef32_pk_bf8_bf16(o, __builtin_bit_cast(v2bf16, d0), scale, false);
-        o = __builtin_amdgcn_cvt_scalef32_pk_bf8_bf16(o, __builtin_bit_cast(v2bf16, d1), scale, true);
-    }
-    return __builtin_bit_cast(uint32_t, o);
-}
 
 template <int FMT>
 __global__ __launch_bounds__(kThreads) void mx_quant_rne8_kernel(const uint8_t* __restrict__ x, uint32_t ld_x_bytes,
