@@ -39,8 +39,9 @@ def log(*a):
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=30,
+                    help="untimed launches first; the launch time keeps falling for about 25 launches after an idle GPU")
     ap.add_argument("--only", type=str, default="", help="comma list of extras: quant,gemm,ffn,fp4,routing,copycal (default: all but copycal)")
     ap.add_argument("--no-extras", action="store_true")
     ap.add_argument("--no-cpu", action="store_true")
@@ -106,19 +107,25 @@ def main() -> int:
     def step():
         ops.mx_gmm_swiglu_quant(a_codes, a_scales, w1, w1s, counts, H, workspace=gws, outs=(act_codes, act_scales))
 
+    # one timed region, measured twice: host clock bracketed by synchronize (-> value) and HIP events recorded on
+    # the launch stream around the same K launches (-> roofline.achieved)
     for _ in range(WARM):
         step()
     torch.cuda.synchronize()
+    ev0 = torch.cuda.Event(enable_timing=True)
+    ev1 = torch.cuda.Event(enable_timing=True)
     t0 = time.perf_counter()
+    ev0.record()
     for _ in range(K_STEPS):
         step()
+    ev1.record()
     torch.cuda.synchronize()
     wall = (time.perf_counter() - t0) / K_STEPS
+    kern = ev0.elapsed_time(ev1) * 1e-3 / K_STEPS
     flop = 2.0 * rows * H * N
     value = flop / wall / 1e12
-    kern = hip_time(step)
     log(f"[gmm1+swiglu+requant cfg3] wall {wall*1e6:.1f} us/step, events {kern*1e6:.1f} us -> {flop/kern/1e12:.0f} TFLOP/s")
-    roofline = {"kernel": "mx_gemm_kernel<E4M3, swiglu+requant epilogue> (grouped, config 3)", "bound": "mfma",
+    roofline = {"kernel": "mx_gemm_pipe_kernel<E4M3, swiglu+requant epilogue, 256x256 tile, 4x1 wavefronts, persistent> (grouped, config 3; one launch also runs the 1-workgroup gmm_prepare_kernel)", "bound": "mfma",
                 "achieved": flop / kern / 1e12, "peak": MXFP8_PEAK_TFLOPS, "unit": "TFLOP/s",
                 "frac": flop / kern / 1e12 / MXFP8_PEAK_TFLOPS, "traffic": None,
                 "flop_per_launch": flop, "avg_launch_us": kern * 1e6}
@@ -184,7 +191,7 @@ def main() -> int:
         tq = hip_time(lambda: lib.cmx_mx_quant(x1.data_ptr(), K1, q1.data_ptr(), K1, s1.data_ptr(), K1 // 32, M1, K1, 0, 0, st),
                       steps=max(K_STEPS, 50))
         bytes_q = M1 * K1 * 2 + M1 * K1 + M1 * K1 // 32
-        extra["mx_quant_cfg1"] = {"kernel": "mx_quant_kernel<E4M3, RNE>", "bound": "hbm", "achieved": bytes_q / tq / 1e9,
+        extra["mx_quant_cfg1"] = {"kernel": "mx_quant_rne8_kernel<E4M3>", "bound": "hbm", "achieved": bytes_q / tq / 1e9,
                                   "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": bytes_q / tq / 1e9 / HBM_PEAK_GBS,
                                   "bytes_per_launch": bytes_q, "avg_launch_us": tq * 1e6, "traffic": None}
         log(f"[mx_quant cfg1] {tq*1e6:.1f} us -> {bytes_q/tq/1e9:.0f} GB/s")
@@ -197,7 +204,7 @@ def main() -> int:
         b2, b2s = ops.mx_quant(torch.randn((N2, K2), generator=g, device=dev).to(torch.bfloat16))
         tg = hip_time(lambda: ops.mx_gemm(a2, a2s, b2, b2s, K2))
         fl2 = 2.0 * M2 * N2 * K2
-        extra["mx_gemm_cfg2"] = {"kernel": "mx_gemm_kernel<E4M3, store epilogue> (dense)", "bound": "mfma",
+        extra["mx_gemm_cfg2"] = {"kernel": "mx_gemm_pipe_kernel<E4M3, store epilogue, 256x256 tile, 2x2 wavefronts> (dense)", "bound": "mfma",
                                  "achieved": fl2 / tg / 1e12, "peak": MXFP8_PEAK_TFLOPS, "unit": "TFLOP/s",
                                  "frac": fl2 / tg / 1e12 / MXFP8_PEAK_TFLOPS, "avg_launch_us": tg * 1e6}
         log(f"[mx_gemm cfg2] {tg*1e6:.1f} us -> {fl2/tg/1e12:.0f} TFLOP/s")
@@ -220,7 +227,7 @@ def main() -> int:
         ws5 = ops.gmm_workspace(E5, dev)
         t5 = hip_time(lambda: ops.mx_gmm(a5, a5s, w5, w5s, c5, K5, "E2M1", "bf16", c=c_out, workspace=ws5))
         fl5 = 2.0 * rows5 * K5 * N5
-        extra["mxfp4_gmm_cfg5"] = {"kernel": "mx_gemm_kernel<E2M1, store epilogue> (grouped)", "bound": "mfma",
+        extra["mxfp4_gmm_cfg5"] = {"kernel": "mx_gemm_dl_kernel<E2M1, store epilogue, 256x256 tile, 8 wavefronts> (grouped)", "bound": "mfma",
                                    "achieved": fl5 / t5 / 1e12, "peak": MXFP4_PEAK_TFLOPS, "unit": "TFLOP/s",
                                    "frac": fl5 / t5 / 1e12 / MXFP4_PEAK_TFLOPS, "avg_launch_us": t5 * 1e6}
         log(f"[mxfp4 gmm cfg5] {t5*1e6:.1f} us -> {fl5/t5/1e12:.0f} TFLOP/s")
