@@ -32,7 +32,9 @@ constexpr int kSlabBytes = 128;     // K bytes per LDS slab and row
 constexpr int kChunks = kSlabBytes / 16;
 constexpr int kXcds = 8;
 
-enum Epilogue { kEpiStore = 0, kEpiSwigluQuant = 1 };
+// kEpiStoreBf16: bf16 output whose rows and row pitch are multiples of four elements (one 8-byte store per
+// accumulator quad, no per-element edge handling): small enough to sit inside a persistent kernel's tile loop
+enum Epilogue { kEpiStore = 0, kEpiSwigluQuant = 1, kEpiStoreBf16 = 2 };
 
 struct GemmParams {
     const uint8_t* a;        // activations codes
@@ -183,7 +185,26 @@ __device__ __forceinline__ void epilogue(const GemmParams& p, const Tile& tc, v1
     const uint32_t l32 = lane & 31u, lh = lane >> 5;
     const uint32_t wt = tc.wt, row0 = tc.row0, rows_valid = tc.rows_valid;
     auto wfrag_row = [&](int f) -> uint32_t { return wfrag_row_of<TW, WW, EPI, FW>(ww, f); };
-    if constexpr (EPI == kEpiStore) {
+    if constexpr (EPI == kEpiStoreBf16) {
+        uint16_t* const c = reinterpret_cast<uint16_t*>(p.c);
+#pragma unroll
+        for (int fm = 0; fm < FM; ++fm) {
+            const uint32_t mloc = wm * (TM / WM) + fm * 32 + l32;
+            if (mloc >= rows_valid) continue;
+            uint16_t* const crow = c + (size_t)(row0 + mloc) * p.ldc;
+#pragma unroll
+            for (int fw = 0; fw < FW; ++fw) {
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    const uint32_t ncol = wt * TW + wfrag_row(fw) + 8 * q + 4 * lh;
+                    if (ncol < p.n)
+                        *reinterpret_cast<uint2*>(crow + ncol) =
+                            make_uint2(cvt_pk_bf16(acc[fw][fm][4 * q], acc[fw][fm][4 * q + 1]),
+                                       cvt_pk_bf16(acc[fw][fm][4 * q + 2], acc[fw][fm][4 * q + 3]));
+                }
+            }
+        }
+    } else if constexpr (EPI == kEpiStore) {
 #pragma unroll
         for (int fm = 0; fm < FM; ++fm) {
             const uint32_t mloc = wm * (TM / WM) + fm * 32 + l32;
@@ -291,7 +312,7 @@ __global__ __launch_bounds__(64 * WW * WM) void mx_gemm_kernel(const GemmParams 
     constexpr int kWLoads = TW / kRowsPerPass;         // 16-byte chunks per thread per slab
     constexpr int kALoads = TM / kRowsPerPass;
     static_assert(FW >= 1 && FM >= 1 && kWLoads >= 1 && kALoads >= 1, "tile too small for the wavefront grid");
-    static_assert(EPI == kEpiStore || (FW % 2 == 0), "gate/up fragments come in pairs");
+    static_assert(EPI != kEpiSwigluQuant || (FW % 2 == 0), "gate/up fragments come in pairs");
     static_assert(TW <= NT && TM <= NT, "one scale row per thread");
     constexpr int kStageBytes = (TW + TM) * kSlabBytes + (TW + TM) * 4 * kScaleDw;
 
@@ -526,7 +547,7 @@ __global__ __launch_bounds__(64 * WW * WM) void mx_gemm_dl_kernel(const GemmPara
     constexpr int kLoadsPerSlab = kTileLoads + kScalePerWave * kScaleDw;
     static_assert(TW % (8 * NW) == 0 && TM % (8 * NW) == 0 && TW % 64 == 0 && TM % 64 == 0, "tile shape");
     static_assert(FW >= 1 && FM >= 1, "tile too small for the wavefront grid");
-    static_assert(EPI == kEpiStore || (FW % 2 == 0), "gate/up fragments come in pairs");
+    static_assert(EPI != kEpiSwigluQuant || (FW % 2 == 0), "gate/up fragments come in pairs");
 
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     uint32_t* const sScale = reinterpret_cast<uint32_t*>(smem + 2 * kSlotBytes);
@@ -840,6 +861,8 @@ TileChoice g_force_tile = {0, 0, 0};   // test/tuning hook: tw == 0 -> heuristic
 // eight-wavefront streaming kernel.
 TileChoice choose_tile(uint32_t m_hint, uint32_t n, int fmt, bool grouped) {
     if (g_force_tile.tw) return g_force_tile;
+    // short problems stream their weights once: the three-slot 256 x 128 kernel keeps two slabs in flight
+    if (m_hint <= 128 && fmt != CMX_FMT_E2M1) return {256, 128, 5};
     if (m_hint <= 64) return {256, 64, 4};
     if (m_hint <= 128) return {256, 128, 8};
     return {256, 256, fmt == CMX_FMT_E2M1 ? 8 : (grouped ? 5 : 4)};
@@ -852,8 +875,17 @@ template <int FMT, int TW, int TM, int EPI>
 int launch_tile(const GemmParams& p, int waves, uint32_t max_m_tiles, hipStream_t s) {
     const bool stream_ok = !g_disable_dl && p.scale_vec && p.kbytes % kSlabBytes == 0;
     if constexpr (TW == 256 && TM == 256 && FMT != CMX_FMT_E2M1) {
-        if (waves == 4 && stream_ok && p.kbytes % (2 * kSlabBytes) == 0) return launch_gemm_pipe<FMT, EPI, 256, 2, 2, 2>(p, max_m_tiles, s);
-        if (waves == 5 && stream_ok && p.kbytes % (2 * kSlabBytes) == 0) return launch_gemm_pipe<FMT, EPI, 256, 4, 1, 2>(p, max_m_tiles, s);
+        if ((waves == 4 || waves == 5) && stream_ok && p.kbytes % (2 * kSlabBytes) == 0) {
+            // plain bf16 output with 4-element-aligned rows takes the lean store epilogue and with it the persistent kernel
+            constexpr int kLean = EPI == kEpiStore ? kEpiStoreBf16 : EPI;
+            const bool lean = EPI == kEpiStore && p.out_type == CMX_OUT_BF16 && p.n % 4 == 0 && p.ldc % 4 == 0 &&
+                              (reinterpret_cast<uintptr_t>(p.c) & 7u) == 0;
+            // (the 4 x 1 layout with the lean store epilogue does not fit the register file without spilling
+            // inside the loop, so the persistent store kernel is always 2 x 2)
+            if (lean) return launch_gemm_pipe<FMT, kLean, 256, 2, 2, 2>(p, max_m_tiles, s);
+            if (waves == 4) return launch_gemm_pipe<FMT, EPI, 256, 2, 2, 2>(p, max_m_tiles, s);
+            return launch_gemm_pipe<FMT, EPI, 256, 4, 1, 2>(p, max_m_tiles, s);
+        }
     }
     if constexpr (TW == 256 && TM == 128 && FMT != CMX_FMT_E2M1) {
         if (waves == 5 && stream_ok) return launch_gemm_pipe<FMT, EPI, 128, 4, 1, 3>(p, max_m_tiles, s);

@@ -107,7 +107,7 @@ __device__ __forceinline__ v8i join8(const v4i& lo, const v4i& hi) {
 //   TM 128, 3 slots, 4 x 1: two slabs instead of one in flight behind the one being consumed, for groups
 //           so short that every tile streams its weights from HBM once and the load latency, not the MFMA
 //           rate, sets the pace.
-__host__ __device__ constexpr bool pipe_is_persistent(int nslot, int epi) { return nslot == 2 && epi == kEpiSwigluQuant; }
+__host__ __device__ constexpr bool pipe_is_persistent(int nslot, int epi) { return nslot == 2 && epi != kEpiStore; }
 
 template <int FMT, int EPI, int TM, int WW, int WM, int NSLOT>
 __global__ __launch_bounds__(256) void mx_gemm_pipe_kernel(const GemmParams p) {
@@ -136,10 +136,11 @@ __global__ __launch_bounds__(256) void mx_gemm_pipe_kernel(const GemmParams p) {
     const uint32_t l32 = lane & 31u, lh = lane >> 5;
 
     // ---- tile sequence of this workgroup ------------------------------------------------------------------
-    // The two-slot kernels with the SwiGLU epilogue are persistent: the grid is one workgroup per CU, and
-    // workgroup j of XCD x walks tiles j, j + (workgroups per XCD), ... of that XCD's contiguous run, carrying
-    // the load pipeline across tile boundaries.  The others take one tile per workgroup (the plain store
-    // epilogue with its three output types and edge cases needs too many registers to sit inside the loop).
+    // The two-slot kernels with the SwiGLU or the lean bf16 store epilogue are persistent: the grid is one
+    // workgroup per CU, and workgroup j of XCD x walks tiles j, j + (workgroups per XCD), ... of that XCD's
+    // contiguous run, carrying the load pipeline across tile boundaries.  The others take one tile per
+    // workgroup (the general store epilogue with its three output types and edge cases needs too many
+    // registers to sit inside the loop).
     constexpr bool kPersistent = pipe_is_persistent(NSLOT, EPI);
     const uint32_t m_tiles_all = count_m_tiles<TM>(p);
     const uint32_t total_tiles = m_tiles_all * p.w_tiles;
