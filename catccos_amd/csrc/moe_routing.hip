@@ -36,8 +36,20 @@ __global__ __launch_bounds__(1024) void route_scan_kernel(uint32_t* __restrict__
     uint32_t* tot = sh;
     uint32_t* part = sh + experts;
     for (uint32_t e = threadIdx.x; e < experts; e += blockDim.x) {
+        // the column walk is latency bound: fetch eight chunk counts at a time before touching the running sum
         uint32_t run = 0;
-        for (uint32_t c = 0; c < chunks; ++c) {
+        uint32_t c = 0;
+        for (; c + 8 <= chunks; c += 8) {
+            uint32_t h[8];
+#pragma unroll
+            for (int i = 0; i < 8; ++i) h[i] = hist[(size_t)(c + i) * experts + e];
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                hist[(size_t)(c + i) * experts + e] = run;
+                run += h[i];
+            }
+        }
+        for (; c < chunks; ++c) {
             const uint32_t h = hist[(size_t)c * experts + e];
             hist[(size_t)c * experts + e] = run;
             run += h;
@@ -68,7 +80,15 @@ __global__ __launch_bounds__(1024) void route_scan_kernel(uint32_t* __restrict__
     __syncthreads();
     for (uint32_t e = threadIdx.x; e < experts; e += blockDim.x) {
         const uint32_t b = tot[e];
-        for (uint32_t c = 0; c < chunks; ++c) hist[(size_t)c * experts + e] += b;
+        uint32_t c = 0;
+        for (; c + 8 <= chunks; c += 8) {
+            uint32_t h[8];
+#pragma unroll
+            for (int i = 0; i < 8; ++i) h[i] = hist[(size_t)(c + i) * experts + e];
+#pragma unroll
+            for (int i = 0; i < 8; ++i) hist[(size_t)(c + i) * experts + e] = h[i] + b;
+        }
+        for (; c < chunks; ++c) hist[(size_t)c * experts + e] += b;
     }
 }
 
@@ -110,12 +130,6 @@ __global__ __launch_bounds__(64) void route_scatter_kernel(const int32_t* __rest
 }
 
 // ---- fused quantise + scatter -------------------------------------------------------------------
-__device__ __forceinline__ uint32_t quad_max(uint32_t v) {
-    uint32_t t = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0xB1, 0xF, 0xF, true);
-    v = v > t ? v : t;
-    t = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x4E, 0xF, 0xF, true);
-    return v > t ? v : t;
-}
 
 // Four lanes per MX block as in the plain quantizer; k % 32 == 0, rows 16-byte aligned.
 __global__ __launch_bounds__(256) void quant_scatter_kernel(const uint16_t* __restrict__ x, uint32_t ld_x,
@@ -132,28 +146,24 @@ __global__ __launch_bounds__(256) void quant_scatter_kernel(const uint16_t* __re
     const uint32_t col = kb * 32 + q * 8;
     uint4 raw = make_uint4(0, 0, 0, 0);
     if (live) raw = *reinterpret_cast<const uint4*>(x + (size_t)row * ld_x + col);
-    uint32_t d[4] = {raw.x, raw.y, raw.z, raw.w};
-    uint32_t amax = 0;
+    // amax, clamp and cast on packed bf16 bit patterns, as in the stand-alone quantizer's fast path
+    const uint32_t d[4] = {raw.x, raw.y, raw.z, raw.w};
+    uint32_t a[4];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        const uint32_t a = d[i] & 0x7FFF7FFFu;
-        const uint32_t lo = a & 0xFFFFu, hi = a >> 16;
-        amax = amax > lo ? amax : lo;
-        amax = amax > hi ? amax : hi;
-    }
-    amax = quad_max(amax);
+    for (int i = 0; i < 4; ++i) a[i] = d[i] & 0x7FFF7FFFu;
+    uint32_t m = pk_max_u16(pk_max_u16(a[0], a[1]), pk_max_u16(a[2], a[3]));
+    m = pk_max_u16(m, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)m, 0xB1, 0xF, 0xF, true));
+    m = pk_max_u16(m, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)m, 0x4E, 0xF, 0xF, true));
+    const uint32_t amax = max(m & 0xFFFFu, m >> 16);
     const int e = block_exp_from_bf16_amax(amax, kEmaxE4M3);
-    float y[8];
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        y[2 * i] = clamp_abs(ldexpf(__uint_as_float(d[i] << 16), -e), 448.0f);
-        y[2 * i + 1] = clamp_abs(ldexpf(__uint_as_float(d[i] & 0xFFFF0000u), -e), 448.0f);
-    }
     if (!live) return;
-    uint32_t w0 = cvt_pk_e4m3(y[0], y[1], 0u, false);
-    w0 = cvt_pk_e4m3(y[2], y[3], w0, true);
-    uint32_t w1 = cvt_pk_e4m3(y[4], y[5], 0u, false);
-    w1 = cvt_pk_e4m3(y[6], y[7], w1, true);
+    const uint32_t lim = (((uint32_t)(e + kEmaxE4M3 + 127) << 7) | 0x60u) * 0x10001u;
+    const float scale = __uint_as_float((uint32_t)(e + 127) << 23);
+    uint32_t c[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) c[i] = pk_min_u16(a[i], lim) | (d[i] & 0x80008000u);
+    const uint32_t w0 = cvt_scaled_pk4<CMX_FMT_E4M3>(c[0], c[1], scale);
+    const uint32_t w1 = cvt_scaled_pk4<CMX_FMT_E4M3>(c[2], c[3], scale);
     const uint8_t sbyte = (uint8_t)(e + 127);
     const bool pad = (kb == nb - 1) && (nb & 1u);
     for (uint32_t r = 0; r < top_k; ++r) {
