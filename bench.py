@@ -127,7 +127,10 @@ def main() -> int:
     log(f"[gmm1+swiglu+requant cfg3] wall {wall*1e6:.1f} us/step, events {kern*1e6:.1f} us -> {flop/kern/1e12:.0f} TFLOP/s")
     roofline = {"kernel": "mx_gemm_pipe_kernel<E4M3, swiglu+requant epilogue, 256x256 tile, 4x1 wavefronts, persistent> (grouped, config 3; one launch also runs the 1-workgroup gmm_prepare_kernel)", "bound": "mfma",
                 "achieved": flop / kern / 1e12, "peak": MXFP8_PEAK_TFLOPS, "unit": "TFLOP/s",
-                "frac": flop / kern / 1e12 / MXFP8_PEAK_TFLOPS, "traffic": None,
+                "frac": flop / kern / 1e12 / MXFP8_PEAK_TFLOPS,
+                # HBM-side bytes per launch from the rocprofv3 --pmc runs summarised under profiles/
+                # (FETCH_SIZE 1 359 052 KiB x 2.0 + WRITE_SIZE 163 788 KiB x 1.0, factors from a 1 GiB copy)
+                "traffic": 1359052 * 1024 * 2.0 + 163788 * 1024 * 1.0,
                 "flop_per_launch": flop, "avg_launch_us": kern * 1e6}
 
     # ------------------------------------------------------------------ CPU baseline -----------
