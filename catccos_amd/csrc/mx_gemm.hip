@@ -137,9 +137,15 @@ __device__ __forceinline__ void decode_tile(const GemmParams& p, uint32_t m_tile
         t.g = lo;
         const uint32_t tp = (uint32_t)p.tile_pref[lo];
         const uint32_t mtg = (uint32_t)p.tile_pref[lo + 1] - tp;
+        // bands of 8 m-tiles share a run of weight tiles (m fastest inside a band): the 32 tiles that an XCD
+        // works on at a time then touch 8 + 4 operand panels instead of mtg + 32/mtg
         const uint32_t local = L - tp * p.w_tiles;
-        t.mt = local % mtg;             // m fastest: neighbours share the weight panel
-        t.wt = local / mtg;
+        const uint32_t band = 8;
+        const uint32_t per_band = band * p.w_tiles;
+        const uint32_t b = local / per_band, within = local % per_band;
+        const uint32_t band_rows = (mtg - b * band) < band ? (mtg - b * band) : band;
+        t.mt = b * band + within % band_rows;
+        t.wt = within / band_rows;
         const uint32_t r_begin = (uint32_t)p.row_off[lo], r_end = (uint32_t)p.row_off[lo + 1];
         t.row0 = r_begin + t.mt * TM;
         t.rows_valid = r_end - t.row0 < (uint32_t)TM ? r_end - t.row0 : (uint32_t)TM;
