@@ -414,7 +414,8 @@ def swiglu_bf16(h_bits) -> np.ndarray:
     h = bf16_bits_to_f32(h_bits)
     half = h.shape[1] // 2
     act, up = h[:, :half], h[:, half:]
-    sig = (np.float32(1.0) / (np.float32(1.0) + np.exp(-act, dtype=np.float32))).astype(np.float32)
+    with np.errstate(over="ignore"):      # exp(-act) = inf for act < -88.7 gives sigmoid 0, the fp32 result
+        sig = (np.float32(1.0) / (np.float32(1.0) + np.exp(-act, dtype=np.float32))).astype(np.float32)
     return f32_to_bf16_bits((act * sig).astype(np.float32) * up)
 
 

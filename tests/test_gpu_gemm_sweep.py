@@ -1,0 +1,69 @@
+"""Seeded shape sweep of the dense and grouped matmuls under the default tile heuristic: every kernel variant
+the dispatcher can pick (hand-scheduled two- and three-slot, streaming, register-staged) against the oracle."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import mx_oracle as O
+from tests.gpu_util import dev, host, close_bf16
+
+pytestmark = pytest.mark.gpu
+
+
+def _shapes(seed, count):
+    rng = np.random.default_rng(seed)
+    out = []
+    for _ in range(count):
+        m = int(rng.choice([1, 17, 64, 100, 128, 129, 255, 256, 257, 300, 511, 600, 777]))
+        n = int(rng.choice([4, 32, 100, 256, 260, 512, 700, 1028]))
+        k = int(rng.choice([32, 96, 128, 256, 384, 512, 768, 1024, 2048]))
+        out.append((m, n, k))
+    return out
+
+
+@pytest.mark.parametrize("m,n,k", _shapes(1, 36))
+def test_dense_sweep(m, n, k):
+    from catccos_amd import ops
+    rng = np.random.default_rng(m * 131 + n * 17 + k)
+    aq, asc = O.mx_quant(O.bf16_round(rng.standard_normal((m, k)).astype(np.float32)), "E4M3")
+    bq, bsc = O.mx_quant(O.bf16_round(rng.standard_normal((n, k)).astype(np.float32)), "E4M3")
+    c = ops.mx_gemm(dev(aq), dev(asc), dev(bq), dev(bsc), k)
+    bad, worst = close_bf16(host(c), O.mx_gemm_f32(aq, asc, bq, bsc))
+    assert bad == 0, (bad, worst)
+
+
+def _groupings(seed, count):
+    rng = np.random.default_rng(seed)
+    out = []
+    for _ in range(count):
+        g = int(rng.integers(1, 9))
+        scale = int(rng.choice([8, 70, 140, 300, 520]))
+        counts = [int(c) for c in rng.integers(0, scale + 1, size=g)]
+        if sum(counts) == 0:
+            counts[0] = 3
+        n = int(rng.choice([64, 256, 320, 768]))
+        k = int(rng.choice([128, 256, 512, 1024]))
+        out.append((tuple(counts), n, k))
+    return out
+
+
+@pytest.mark.parametrize("counts,n,k", _groupings(2, 24))
+def test_grouped_sweep(counts, n, k):
+    from catccos_amd import ops
+    rng = np.random.default_rng(sum(counts) * 7 + n + k)
+    m = sum(counts)
+    aq, asc = O.mx_quant(O.bf16_round(rng.standard_normal((m, k)).astype(np.float32)))
+    ws_ = [O.mx_quant(O.bf16_round(rng.standard_normal((n, k)).astype(np.float32)), "E4M3", "lut") for _ in counts]
+    wq, ws = np.stack([q for q, _ in ws_]), np.stack([s for _, s in ws_])
+    cnt = dev(np.array(counts, dtype=np.int32))
+    c = ops.mx_gmm(dev(aq), dev(asc), dev(wq), dev(ws), cnt, k)
+    bad, worst = close_bf16(host(c), O.mx_gmm_f32(aq, asc, wq, ws, list(counts)))
+    assert bad == 0, (bad, worst)
+    if n % 64 == 0:
+        # fused SwiGLU + requant on the same operands: dequantised activation within the bound of two chained
+        # bf16 roundings and one E4M3 quantisation step
+        codes, scales, _ = ops.mx_gmm_swiglu_quant(dev(aq), dev(asc), dev(wq), dev(ws), cnt, k)
+        _, _, gq, gs = O.gmm1_swiglu_quant(aq, asc, wq, ws, list(counts))
+        deq, deq_g = O.mx_dequant(host(codes), host(scales)), O.mx_dequant(gq, gs)
+        bound = 0.13 * np.abs(deq_g) + 2.0 ** -5 * np.abs(deq_g).max(axis=1, keepdims=True) + 1e-6
+        assert np.all(np.abs(deq - deq_g) <= bound)
