@@ -1,0 +1,148 @@
+"""The BASELINE configurations at their full sizes: sampled rows against the oracle plus properties that
+do not depend on the size (exact scale linearity, row-permutation equivariance, gate-weight linearity).
+Inputs are generated and quantised on the GPU; only the sampled rows travel to the host for the oracle."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import mx_oracle as O
+from catccos_amd import workloads as W
+from tests.gpu_util import host, close_bf16
+
+pytestmark = pytest.mark.gpu
+
+
+def _gpu_mx(shape, seed, std=1.0, fmt="E4M3", mode="rne"):
+    from catccos_amd import ops
+    g = torch.Generator(device="cuda")
+    g.manual_seed(seed)
+    x = (torch.randn(shape, generator=g, device="cuda") * std).to(torch.bfloat16)
+    return ops.mx_quant(x, fmt, mode)
+
+
+def _np(t):
+    return t.cpu().numpy()
+
+
+def test_config2_dense_full_size():
+    from catccos_amd import ops
+    M, N, K = 8192, 4096, 7168
+    a, a_s = _gpu_mx((M, K), 21)
+    b, b_s = _gpu_mx((N, K), 22)
+    c = ops.mx_gemm(a, a_s, b, b_s, K)
+    rows = np.array([0, 1, 255, 256, 257, 4095, 4096, 8190, 8191] + list(np.random.default_rng(0).integers(0, M, 23)))
+    gold = O.mx_gemm_f32(_np(a[rows]), _np(a_s[rows]), _np(b), _np(b_s))
+    bad, worst = close_bf16(host(c[rows]), gold)
+    assert bad == 0, (bad, worst)
+    # one more on every activation scale doubles every product and every partial sum: the bf16 result doubles exactly
+    c2 = ops.mx_gemm(a, a_s + 1, b, b_s, K)
+    assert torch.equal(c2.float(), c.float() * 2)
+    # permuting activation rows permutes result rows bit for bit (a row's sums do not depend on its tile)
+    perm = torch.randperm(M, device="cuda", generator=torch.Generator(device="cuda").manual_seed(3))
+    cp = ops.mx_gemm(a[perm].contiguous(), a_s[perm].contiguous(), b, b_s, K)
+    assert torch.equal(cp, c[perm])
+
+
+def test_config3_gmm1_swiglu_requant_full_size():
+    from catccos_amd import ops
+    E, T, TOPK, K, N = 16, 4096, 8, 7168, 4096
+    idx = W.zipf_routing(T, E, TOPK, 3)
+    counts = np.bincount(idx.reshape(-1), minlength=E).astype(np.int32)
+    rows = int(counts.sum())
+    a, a_s = _gpu_mx((rows, K), 31)
+    w = torch.empty((E, N, K), dtype=torch.uint8, device="cuda")
+    w_s = torch.empty((E, N, K // 32), dtype=torch.uint8, device="cuda")
+    for e in range(E):
+        w[e], w_s[e] = _gpu_mx((N, K), 100 + e, std=0.02, mode="lut")
+    cnt = torch.from_numpy(counts).cuda()
+    codes, scales, _ = ops.mx_gmm_swiglu_quant(a, a_s, w, w_s, cnt, K)
+    off = np.concatenate([[0], np.cumsum(counts)])
+    rng = np.random.default_rng(1)
+    for e in [int(np.argmax(counts)), int(np.argmin(np.where(counts > 0, counts, 1 << 30))), 5]:
+        if counts[e] == 0:
+            continue
+        pick = np.unique(np.concatenate([[0, counts[e] - 1], rng.integers(0, counts[e], 6)])) + off[e]
+        _, _, gq, gs = O.gmm1_swiglu_quant(_np(a[pick]), _np(a_s[pick]), _np(w[e:e + 1]), _np(w_s[e:e + 1]), [len(pick)])
+        deq, deq_g = O.mx_dequant(_np(codes[pick]), _np(scales[pick])), O.mx_dequant(gq, gs)
+        bound = 0.13 * np.abs(deq_g) + 2.0 ** -5 * np.abs(deq_g).max(axis=1, keepdims=True) + 1e-9
+        assert np.all(np.abs(deq - deq_g) <= bound), e
+    # every scale byte is a legal E8M0 value and no code is the E4M3 NaN pattern
+    assert int((codes & 0x7F).eq(0x7F).sum()) == 0
+    # group-order equivariance: the same rows as groups in reverse expert order give the same codes per row
+    order = list(range(E - 1, -1, -1))
+    src = torch.cat([torch.arange(off[e], off[e + 1], device="cuda") for e in order])
+    codes_r, scales_r, _ = ops.mx_gmm_swiglu_quant(a[src].contiguous(), a_s[src].contiguous(), w[order].contiguous(),
+                                                  w_s[order].contiguous(), torch.from_numpy(counts[order].copy()).cuda(), K)
+    assert torch.equal(codes_r, codes[src]) and torch.equal(scales_r, scales[src])
+
+
+def test_config5_fp4_gmm_full_size():
+    from catccos_amd import ops
+    E, T, K, N = 32, 8192, 7168, 4096
+    idx = W.zipf_routing(T, E, 8, 8)
+    counts = np.bincount(idx.reshape(-1), minlength=E).astype(np.int32)
+    rows = int(counts.sum())
+    g = torch.Generator(device="cuda")
+    g.manual_seed(51)
+    a, a_s = ops.mx_quant((torch.rand((rows, K), generator=g, device="cuda") * 4 - 2).to(torch.bfloat16), "E2M1", "lut")
+    w = torch.empty((E, N, K // 2), dtype=torch.uint8, device="cuda")
+    w_s = torch.empty((E, N, K // 32), dtype=torch.uint8, device="cuda")
+    for e in range(E):
+        w[e], w_s[e] = ops.mx_quant((torch.rand((N, K), generator=g, device="cuda") * 4 - 2).to(torch.bfloat16), "E2M1", "lut")
+    c = ops.mx_gmm(a, a_s, w, w_s, torch.from_numpy(counts).cuda(), K, "E2M1", "bf16")
+    off = np.concatenate([[0], np.cumsum(counts)])
+    rng = np.random.default_rng(2)
+    for e in [int(np.argmax(counts)), 7]:
+        if counts[e] == 0:
+            continue
+        pick = np.unique(np.concatenate([[0, counts[e] - 1], rng.integers(0, counts[e], 6)])) + off[e]
+        gold = O.mx_gmm_f32(O.unpack_fp4(_np(a[pick])), _np(a_s[pick]), O.unpack_fp4(_np(w[e:e + 1])), _np(w_s[e:e + 1]), [len(pick)],
+                            "E2M1", "E2M1")
+        bad, worst = close_bf16(host(c[pick]), gold, rtol=1e-2, atol=5e-2)
+        assert bad == 0, (e, bad, worst)
+    c2 = ops.mx_gmm(a, a_s + 1, w, w_s, torch.from_numpy(counts).cuda(), K, "E2M1", "bf16")
+    assert torch.equal(c2.float(), c.float() * 2)
+
+
+def test_config4_ffn_full_size():
+    from catccos_amd import ops
+    T, E, TOPK, K, N = 8192, 256, 8, 7168, 4096
+    idx_h, p_h = W.softmax_topk_routing(T, E, TOPK, 41)
+    idx, p = torch.from_numpy(idx_h.astype(np.int32)).cuda(), torch.from_numpy(p_h.astype(np.float32)).cuda()
+    g = torch.Generator(device="cuda")
+    g.manual_seed(42)
+    x = torch.randn((T, K), generator=g, device="cuda").to(torch.bfloat16)
+    w1 = torch.empty((E, N, K), dtype=torch.uint8, device="cuda")
+    w1s = torch.empty((E, N, K // 32), dtype=torch.uint8, device="cuda")
+    w2 = torch.empty((E, K, N // 2), dtype=torch.uint8, device="cuda")
+    w2s = torch.empty((E, K, N // 64), dtype=torch.uint8, device="cuda")
+    for e in range(E):
+        w1[e], w1s[e] = _gpu_mx((N, K), 1000 + e, std=0.02, mode="lut")
+        w2[e], w2s[e] = _gpu_mx((K, N // 2), 2000 + e, std=0.02, mode="lut")
+    ws = torch.full((ops.ffn_workspace_bytes(T, K, N, E, TOPK),), 0xA5, dtype=torch.uint8, device="cuda")
+    out = ops.dispatch_ffn_combine(x, idx, p, w1, w1s, w2, w2s, workspace=ws)
+    # sampled tokens against the oracle chain restricted to their own experts (re-labelled 0..n-1)
+    toks = np.array([0, 4097, 8191])
+    used = np.unique(idx_h[toks])
+    relabel = {int(e): i for i, e in enumerate(used)}
+    sub_idx = np.vectorize(relabel.get)(idx_h[toks]).astype(np.int32)
+    used_t = torch.from_numpy(used).cuda()
+    gold = O.bf16_bits_to_f32(O.moe_ffn(host(x[toks]), sub_idx, p_h[toks].astype(np.float32), _np(w1[used_t]), _np(w1s[used_t]),
+                                        _np(w2[used_t]), _np(w2s[used_t])))
+    got = O.bf16_bits_to_f32(host(out[toks]))
+    diff = np.abs(got - gold)
+    assert (diff > 1e-2 + 1e-2 * np.abs(gold)).sum() <= got.size // 500 and diff.max() <= 5e-2, (diff.max(),)
+    # routing tables at full size: a permutation, keys non-decreasing, stable within a key
+    lay = ops.ffn_workspace_layout(T, K, N, E, TOPK)
+    rows = T * TOPK
+    s2s = ws[lay["sorted2src"]:lay["sorted2src"] + rows * 4].view(torch.int32)
+    src2 = ws[lay["src2sorted"]:lay["src2sorted"] + rows * 4].view(torch.int32)
+    keys = idx.reshape(-1)[s2s.long()]
+    assert torch.equal(torch.sort(s2s).values, torch.arange(rows, device="cuda", dtype=torch.int32))
+    assert bool((keys[1:] >= keys[:-1]).all())
+    same = keys[1:] == keys[:-1]
+    assert bool((s2s[1:][same] > s2s[:-1][same]).all())
+    assert torch.equal(src2[s2s.long()], torch.arange(rows, device="cuda", dtype=torch.int32))
+    # doubling every gate weight doubles the bf16 output exactly (the combine multiplies, then adds in fp32)
+    out2 = ops.dispatch_ffn_combine(x, idx, p * 2, w1, w1s, w2, w2s, workspace=ws)
+    assert torch.equal(out2.float(), out.float() * 2)
