@@ -754,24 +754,44 @@ __global__ __launch_bounds__(64 * WW * WM) void mx_gemm_dl_kernel(const GemmPara
 
 #include "mx_gemm_pipe.h"
 
-// Row offsets and m-tile prefix of the groups (one workgroup).
-__global__ void gmm_prepare_kernel(const int32_t* __restrict__ sizes, uint32_t groups, uint32_t tile_m,
-                                   int32_t* __restrict__ row_off, int32_t* __restrict__ tile_pref,
-                                   int32_t* __restrict__ tile_ctr) {
-    extern __shared__ int32_t sh[];
+// Row offsets and m-tile prefix of the groups (one workgroup of 256 threads): each thread sums a contiguous
+// run of groups, the 256 partial sums are scanned in LDS, and each thread writes its run.
+__global__ __launch_bounds__(256) void gmm_prepare_kernel(const int32_t* __restrict__ sizes, uint32_t groups, uint32_t tile_m,
+                                                           int32_t* __restrict__ row_off, int32_t* __restrict__ tile_pref,
+                                                           int32_t* __restrict__ tile_ctr) {
+    __shared__ int32_t part_r[256], part_t[256];
     if (threadIdx.x < kXcds) tile_ctr[threadIdx.x] = 0;
-    for (uint32_t i = threadIdx.x; i < groups; i += blockDim.x) sh[i] = sizes[i] > 0 ? sizes[i] : 0;
+    const uint32_t per = (groups + 255) / 256;
+    const uint32_t lo = threadIdx.x * per, hi = lo + per < groups ? lo + per : groups;
+    int32_t r = 0, t = 0;
+    for (uint32_t i = lo; i < hi; ++i) {
+        const int32_t c = sizes[i] > 0 ? sizes[i] : 0;
+        r += c;
+        t += (c + (int32_t)tile_m - 1) / (int32_t)tile_m;
+    }
+    part_r[threadIdx.x] = r;
+    part_t[threadIdx.x] = t;
     __syncthreads();
-    if (threadIdx.x == 0) {
-        int32_t r = 0, t = 0;
-        for (uint32_t i = 0; i < groups; ++i) {
-            row_off[i] = r;
-            tile_pref[i] = t;
-            r += sh[i];
-            t += (sh[i] + (int32_t)tile_m - 1) / (int32_t)tile_m;
-        }
-        row_off[groups] = r;
-        tile_pref[groups] = t;
+    for (uint32_t d = 1; d < 256; d <<= 1) {
+        const int32_t vr = threadIdx.x >= d ? part_r[threadIdx.x - d] : 0;
+        const int32_t vt = threadIdx.x >= d ? part_t[threadIdx.x - d] : 0;
+        __syncthreads();
+        part_r[threadIdx.x] += vr;
+        part_t[threadIdx.x] += vt;
+        __syncthreads();
+    }
+    r = threadIdx.x ? part_r[threadIdx.x - 1] : 0;
+    t = threadIdx.x ? part_t[threadIdx.x - 1] : 0;
+    for (uint32_t i = lo; i < hi; ++i) {
+        const int32_t c = sizes[i] > 0 ? sizes[i] : 0;
+        row_off[i] = r;
+        tile_pref[i] = t;
+        r += c;
+        t += (c + (int32_t)tile_m - 1) / (int32_t)tile_m;
+    }
+    if (threadIdx.x == 255) {
+        row_off[groups] = part_r[255];
+        tile_pref[groups] = part_t[255];
     }
 }
 
@@ -992,8 +1012,8 @@ int gmm_common(GemmParams& p, const int32_t* group_sizes, uint32_t groups, uint3
     int32_t* row_off = static_cast<int32_t*>(workspace);
     int32_t* tile_pref = row_off + (groups + 1);
     int32_t* tile_ctr = tile_pref + (groups + 1);
-    hipLaunchKernelGGL(gmm_prepare_kernel, dim3(1), dim3(256), groups * sizeof(int32_t), s, group_sizes, groups,
-                       (uint32_t)t.tm, row_off, tile_pref, tile_ctr);
+    hipLaunchKernelGGL(gmm_prepare_kernel, dim3(1), dim3(256), 0, s, group_sizes, groups, (uint32_t)t.tm, row_off, tile_pref,
+                       tile_ctr);
     CMX_LAUNCH_CHECK();
     p.row_off = row_off;
     p.tile_pref = tile_pref;
