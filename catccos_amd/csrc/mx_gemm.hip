@@ -833,7 +833,8 @@ int launch_gemm_dl(const GemmParams& p, uint32_t max_m_tiles, hipStream_t s) {
 
 template <int FMT, int EPI, int TM, int WW, int WM, int NSLOT>
 int launch_gemm_pipe(const GemmParams& p, uint32_t max_m_tiles, hipStream_t s) {
-    constexpr size_t smem = NSLOT * (256 + TM) * (kSlabBytes + 4) + 16;     // ring, scale ring, next-tile mailbox
+    // tile ring, scale ring (two-slot kernels: two blocks of 16 bytes per row), next-tile mailbox
+    constexpr size_t smem = NSLOT * (256 + TM) * kSlabBytes + (NSLOT == 2 ? 2 * (256 + TM) * 16 : NSLOT * (256 + TM) * 4) + 16;
     auto kfn = mx_gemm_pipe_kernel<FMT, EPI, TM, WW, WM, NSLOT>;
     static bool attr_set = false;
     if (!attr_set) {
@@ -901,7 +902,10 @@ template <int FMT, int TW, int TM, int EPI>
 int launch_tile(const GemmParams& p, int waves, uint32_t max_m_tiles, hipStream_t s) {
     const bool stream_ok = !g_disable_dl && p.scale_vec && p.kbytes % kSlabBytes == 0;
     if constexpr (TW == 256 && TM == 256 && FMT != CMX_FMT_E2M1) {
-        if ((waves == 4 || waves == 5) && stream_ok && p.kbytes % (2 * kSlabBytes) == 0) {
+        // whole four-slab scale blocks, fetched 16 bytes per row: K a multiple of 512 bytes, 16-byte aligned scale rows
+        const bool sc16 = p.ld_as % 16 == 0 && p.ld_ws % 16 == 0 && (reinterpret_cast<uintptr_t>(p.a_scale) & 15u) == 0 &&
+                          (reinterpret_cast<uintptr_t>(p.w_scale) & 15u) == 0;
+        if ((waves == 4 || waves == 5) && stream_ok && sc16 && p.kbytes % (4 * kSlabBytes) == 0) {
             // plain bf16 output with 4-element-aligned rows takes the lean store epilogue and with it the persistent kernel
             constexpr int kLean = EPI == kEpiStore ? kEpiStoreBf16 : EPI;
             const bool lean = EPI == kEpiStore && p.out_type == CMX_OUT_BF16 && p.n % 4 == 0 && p.ldc % 4 == 0 &&

@@ -121,10 +121,16 @@ __global__ __launch_bounds__(256) void mx_gemm_pipe_kernel(const GemmParams p) {
     constexpr int kRows = TW + TM;
     constexpr int kSlotBytes = kRows * kSlabBytes;            // 64 KiB or 48 KiB
     constexpr int kScaleBase = NSLOT * kSlotBytes;            // scale ring behind the tile slots
-    constexpr int kScaleSlotBytes = kRows * 4;
+    // Two-slot kernels fetch the scales of FOUR slabs at a time (16 bytes per row, one load per 64 rows): a scale
+    // load touches a different cache line in every lane, so one load per slab would pull as many lines through
+    // the vector L1 as the tile data itself.  Their scale ring holds two such blocks, [block][row][4 dwords].
+    // The three-slot kernel keeps one dword per row and slab, [slot][row].
+    constexpr bool kSc4 = NSLOT == 2;
+    constexpr int kScaleSlotBytes = kSc4 ? kRows * 16 : kRows * 4;
+    constexpr int kScaleRingBytes = kSc4 ? 2 * kScaleSlotBytes : NSLOT * kScaleSlotBytes;
     constexpr int kTileLoads = kRows / (8 * NW);              // LDS-DMA loads per wavefront and slab (16 or 12)
     constexpr int kWTileLoads = TW / (8 * NW);                // the first 8 fetch weight rows
-    constexpr int kLoadsPerSlab = kTileLoads + 2;             // plus one weight and one activation scale load
+    constexpr int kLoadsPerSlab = kTileLoads + 2;             // three-slot kernel: plus one weight and one activation scale load
 
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t*)smem;
@@ -207,18 +213,33 @@ __global__ __launch_bounds__(256) void mx_gemm_pipe_kernel(const GemmParams p) {
     aim_loads_at(tile_id);
     Tile tc = tq;                               // tile of the MFMA stream / epilogue
 
-    const uint32_t nslab = p.kbytes / kSlabBytes;
+    auto nslab_of = [](const GemmParams& q) -> uint32_t { return q.kbytes / kSlabBytes; };
+    const uint32_t nslab = nslab_of(p);
     const uint32_t dma_base = __builtin_amdgcn_readfirstlane(lds0 + wave * 1024);
-    const uint32_t sdma_base = __builtin_amdgcn_readfirstlane(lds0 + kScaleBase + wave * 256);
-    const uint32_t sdma_base_a = __builtin_amdgcn_readfirstlane(lds0 + kScaleBase + TW * 4 + sa_blk * 256);
+    constexpr int kScaleRowBytes = kSc4 ? 16 : 4;
+    const uint32_t sdma_base = __builtin_amdgcn_readfirstlane(lds0 + kScaleBase + wave * 64 * kScaleRowBytes);
+    const uint32_t sdma_base_a = __builtin_amdgcn_readfirstlane(lds0 + kScaleBase + (TW + sa_blk * 64) * kScaleRowBytes);
 
     auto issue_tile_load = [&](int slot, int i, uint32_t koff) {
         dma_b128(dma_base + slot * kSlotBytes + i * (NW * 1024), goff[i], i < kWTileLoads ? w_rs : a_rs, koff);
     };
-    auto issue_scale_loads = [&](int slot, uint32_t soff) {
+    auto issue_scale_loads = [&](int slot, uint32_t soff) {          // one slab (three-slot kernel)
         dma_b32(sdma_base + slot * kScaleSlotBytes, sgoff_w, ws_rs, soff);
         dma_b32(sdma_base_a + slot * kScaleSlotBytes, sgoff_a, as_rs, soff);
     };
+    // four slabs: block `blk` of the load stream's tile into ring position `pos` (0/1)
+    uint32_t blocks_issued = 0;          // running count over all tiles of this workgroup: ring position = count & 1
+    auto issue_scale_block = [&](uint32_t blk) {
+        const uint32_t pos = blocks_issued & 1u;
+        ++blocks_issued;
+        dma_b128(sdma_base + pos * kScaleSlotBytes, sgoff_w, ws_rs, blk * 16);
+        dma_b128(sdma_base_a + pos * kScaleSlotBytes, sgoff_a, as_rs, blk * 16);
+    };
+    // the load stream is at slab q of its tile: block 0 goes out with slab 0, block b+1 with slab 4b+1 (the ring
+    // position it takes was last read one slab earlier)
+    const uint32_t nblk = nslab_of(p) / 4;
+    auto scale_block_due = [&](uint32_t q) -> bool { return q == 0 || ((q & 3u) == 1u && (q >> 2) + 1 < nblk); };
+    auto scale_block_of = [&](uint32_t q) -> uint32_t { return q == 0 ? 0u : (q >> 2) + 1; };
     auto clamp_slab = [&](uint32_t slab) -> uint32_t { return slab < nslab ? slab : nslab - 1; };   // past the end: harmless reload
 
     // ---- fragment read addresses ------------------------------------------------------------------
@@ -235,8 +256,14 @@ __global__ __launch_bounds__(256) void mx_gemm_pipe_kernel(const GemmParams p) {
             wb[s][j] = lds0 + s * kSlotBytes + (w_row_base + l32) * kSlabBytes + ch;
             ab[s][j] = lds0 + s * kSlotBytes + (TW + wm * (TM / WM) + l32) * kSlabBytes + ch;
         }
-    const uint32_t swb = lds0 + kScaleBase + (w_row_base + l32) * 4;
-    const uint32_t sab = lds0 + kScaleBase + (TW + wm * (TM / WM) + l32) * 4;
+    const uint32_t swb = lds0 + kScaleBase + (w_row_base + l32) * kScaleRowBytes;
+    const uint32_t sab = lds0 + kScaleBase + (TW + wm * (TM / WM) + l32) * kScaleRowBytes;
+    // two-slot kernels: running index (over all tiles) of the slab whose scales are read next; its block sits
+    // at ring position (index / 4) & 1, its dword at index & 3
+    uint32_t scale_read_slab = 0;
+    auto scale_read_offset = [&]() -> uint32_t {
+        return __builtin_amdgcn_readfirstlane(((scale_read_slab >> 2) & 1u) * kScaleSlotBytes + (scale_read_slab & 3u) * 4);
+    };
     const uint32_t sshift = 8 * lh;
 
     v16f acc[FW][FM];
@@ -267,12 +294,21 @@ __global__ __launch_bounds__(256) void mx_gemm_pipe_kernel(const GemmParams p) {
         read_half(slot_c, step_c, std::integral_constant<int, 2 * pos>{}, flo, fhi);
         read_half(slot_c, step_c, std::integral_constant<int, 2 * pos + 1>{}, flo, fhi);
     };
-    auto read_scale = [&](auto slot_c, auto idx_c) {
+    auto read_scale = [&](auto slot_c, auto idx_c) {                 // three-slot kernel: [slot][row]
         constexpr int slot = decltype(slot_c)::value, idx = decltype(idx_c)::value;
         if constexpr (idx < FW)
             sraw[idx] = lds_read_b32<slot * kScaleSlotBytes + CMX_PIPE_WOFF(idx) * 4>(swb);
         else
             sraw[idx] = lds_read_b32<slot * kScaleSlotBytes + (idx - FW) * 32 * 4>(sab);
+    };
+    // two-slot kernels: swb_at / sab_at = base + ring position and dword of the slab being read
+    auto read_scale_at = [&](uint32_t swb_at, uint32_t sab_at, auto idx_c) {
+        constexpr int idx = decltype(idx_c)::value;
+        (void)sraw;
+        if constexpr (idx < FW)
+            sraw[idx] = lds_read_b32<CMX_PIPE_WOFF(idx) * 16>(swb_at);
+        else
+            sraw[idx] = lds_read_b32<(idx - FW) * 32 * 16>(sab_at);
     };
 
     using I0 = std::integral_constant<int, 0>;
@@ -280,7 +316,24 @@ __global__ __launch_bounds__(256) void mx_gemm_pipe_kernel(const GemmParams p) {
     using I2 = std::integral_constant<int, 2>;
 
     // ---- prologue: fill the ring, wait for slab 0 -------------------------------------------------------
-    {
+    if constexpr (kSc4) {
+        // scale blocks first, so that the wait below can leave exactly the 16 tile loads of slab 1 in flight
+        issue_scale_block(0);
+        if (nblk > 1) issue_scale_block(1);
+#pragma unroll
+        for (int i = 0; i < kTileLoads; ++i) issue_tile_load(0, i, 0);
+        const uint32_t k1 = clamp_slab(1);
+#pragma unroll
+        for (int i = 0; i < kTileLoads; ++i) issue_tile_load(1, i, k1 * kSlabBytes);
+        asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(kTileLoads) : "memory");      // slab 0 and its scales have landed everywhere
+        static_for<0, NF>([&](auto ic) { read_frag(I0{}, I0{}, ic, f0lo, f0hi); });
+        {
+            const uint32_t off = scale_read_offset();
+            const uint32_t swb_at = swb + off, sab_at = sab + off;
+            static_for<0, NF>([&](auto ic) { read_scale_at(swb_at, sab_at, ic); });
+            ++scale_read_slab;
+        }
+    } else {
         static_for<0, NSLOT>([&](auto sc) {
             constexpr int slot = decltype(sc)::value;
             const uint32_t k = clamp_slab(slot);
@@ -329,13 +382,15 @@ __global__ __launch_bounds__(256) void mx_gemm_pipe_kernel(const GemmParams p) {
         for (int i = 0; i < NF; ++i) asm volatile("" ::"v"(scur[set][i]));
     };
     constexpr int kReads = 2 * NF;
+    constexpr uint32_t kNoSlab = 0xFFFFFFFFu;
 
     // ---- two-slot ring -------------------------------------------------------------------------------------
     // One slab; SLOT = ring slot of slab s (compile-time so that every LDS offset is an immediate).  On entry
     // fragment set 0 and the shifted scales of the slab are in registers.  kR reads go behind each of the first
     // MFMAs of a step; after MFMA kB1 the last of them has had time to land; kEarly tile loads of slab s+2
     // are issued already in step 0, behind the first barrier.
-    auto slab_body2 = [&](auto slot_c, uint32_t koff, uint32_t soff) {
+    // q = slab of the load stream within its tile (kNoSlab: nothing new to request, re-request slab koff)
+    auto slab_body2 = [&](auto slot_c, uint32_t koff, uint32_t q) {
         constexpr int slot = decltype(slot_c)::value;
         constexpr int kR = NF > 8 ? 3 : 2;
         constexpr int kB1 = (kReads + kR - 1) / kR;
@@ -344,6 +399,9 @@ __global__ __launch_bounds__(256) void mx_gemm_pipe_kernel(const GemmParams p) {
         static_assert(kM == 16 && kB1 + kScaleMfmas + 1 <= 14, "the scale shift must sit at least two MFMAs before the end of the step");
         using SlotT = std::integral_constant<int, slot>;
         using OtherT = std::integral_constant<int, slot ^ 1>;
+        const uint32_t sc_off = scale_read_offset();             // where the scales of the next slab sit
+        const uint32_t swb_at = swb + sc_off, sab_at = sab + sc_off;
+        ++scale_read_slab;
         // ---- step 0 ----
         static_for<0, kM>([&](auto ic) {
             constexpr int i = decltype(ic)::value;
@@ -365,14 +423,16 @@ __global__ __launch_bounds__(256) void mx_gemm_pipe_kernel(const GemmParams p) {
             constexpr int i = decltype(ic)::value;
             step_mfma(I2{}, ic, f1lo, f1hi, SlotT{});
             if constexpr (i + kEarly < kTileLoads) issue_tile_load(slot, i + kEarly, koff);
-            if constexpr (i + kEarly == kTileLoads) issue_scale_loads(slot, soff);
+            if constexpr (i + kEarly == kTileLoads) {
+                if (q != kNoSlab && scale_block_due(q)) issue_scale_block(scale_block_of(q));
+            }
             static_for<0, kR>([&](auto jc) {
                 constexpr int r = i * kR + decltype(jc)::value;
                 if constexpr (r < kReads) read_half(OtherT{}, I0{}, std::integral_constant<int, r>{}, f0lo, f0hi);
             });
             if constexpr (i >= kB1 && i < kB1 + kScaleMfmas) {
-                read_scale(OtherT{}, std::integral_constant<int, 2 * (i - kB1)>{});
-                if constexpr (2 * (i - kB1) + 1 < NF) read_scale(OtherT{}, std::integral_constant<int, 2 * (i - kB1) + 1>{});
+                read_scale_at(swb_at, sab_at, std::integral_constant<int, 2 * (i - kB1)>{});
+                if constexpr (2 * (i - kB1) + 1 < NF) read_scale_at(swb_at, sab_at, std::integral_constant<int, 2 * (i - kB1) + 1>{});
             }
             if constexpr (i == kB1 + kScaleMfmas + 1) {
                 asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
@@ -462,16 +522,16 @@ __global__ __launch_bounds__(256) void mx_gemm_pipe_kernel(const GemmParams p) {
         fence_accumulators();
         epilogue<TW, TM, WW, WM, EPI, FW, FM>(p, tc, acc, ww, wm, lane);
     } else if constexpr (!kPersistent) {
-        for (uint32_t s = 0; s < nslab; s += 2) {      // the host only selects this kernel for an even slab count
-            const uint32_t q0 = clamp_slab(s + 2), q1 = clamp_slab(s + 3);
-            slab_body2(I0{}, q0 * kSlabBytes, q0 * 4);
-            slab_body2(I1{}, q1 * kSlabBytes, q1 * 4);
+        for (uint32_t s = 0; s < nslab; s += 2) {      // the host only selects this kernel for a slab count that is a multiple of four
+            const uint32_t q0 = s + 2, q1 = s + 3;
+            slab_body2(I0{}, clamp_slab(q0) * kSlabBytes, q0 < nslab ? q0 : kNoSlab);
+            slab_body2(I1{}, clamp_slab(q1) * kSlabBytes, q1 < nslab ? q1 : kNoSlab);
         }
         asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
         fence_accumulators();
         epilogue<TW, TM, WW, WM, EPI, FW, FM>(p, tc, acc, ww, wm, lane);
     } else {
-        // The host only selects this kernel for an even slab count.  The load stream runs two slabs ahead of
+        // The host only selects this kernel for a slab count that is a multiple of four.  The load stream runs two slabs ahead of
         // the MFMA stream: when it reaches the end of the tile it is aimed at the workgroup's next tile (or keeps
         // re-requesting the last slab when there is none), so the loads and the fragment reads run on through
         // the tile boundary and only the epilogue and the clearing of the accumulators interrupt the MFMAs.
@@ -485,7 +545,7 @@ __global__ __launch_bounds__(256) void mx_gemm_pipe_kernel(const GemmParams p) {
         for (;;) {
             if (sq == nslab) {
                 if (p.tile_ctr != nullptr) {
-                    uint32_t* const mailbox = reinterpret_cast<uint32_t*>(smem + kScaleBase + NSLOT * kScaleSlotBytes);
+                    uint32_t* const mailbox = reinterpret_cast<uint32_t*>(smem + kScaleBase + kScaleRingBytes);
                     if (tid == 0) *mailbox = atomicAdd(reinterpret_cast<unsigned int*>(p.tile_ctr) + blockIdx.x % kXcds, 1u);
                     __syncthreads();
                     next_id = run_first + tile_stride + __builtin_amdgcn_readfirstlane(*mailbox);
@@ -498,9 +558,8 @@ __global__ __launch_bounds__(256) void mx_gemm_pipe_kernel(const GemmParams p) {
                     sq = 0;
                 }
             }
-            const uint32_t q0 = clamp_slab(sq), q1 = clamp_slab(sq + 1);
-            slab_body2(I0{}, q0 * kSlabBytes, q0 * 4);
-            slab_body2(I1{}, q1 * kSlabBytes, q1 * 4);
+            slab_body2(I0{}, clamp_slab(sq) * kSlabBytes, sq < nslab ? sq : kNoSlab);
+            slab_body2(I1{}, clamp_slab(sq + 1) * kSlabBytes, sq + 1 < nslab ? sq + 1 : kNoSlab);
             sq += 2;
             sm += 2;
             if (sm == nslab) {
@@ -522,7 +581,13 @@ __global__ __launch_bounds__(256) void mx_gemm_pipe_kernel(const GemmParams p) {
                 // The last slab has already read the new tile's first fragments and scales, but carrying them
                 // through the epilogue costs more registers than there are: read them again (slot 0, landed).
                 static_for<0, NF>([&](auto ic) { read_frag(I0{}, I0{}, ic, f0lo, f0hi); });
-                static_for<0, NF>([&](auto ic) { read_scale(I0{}, ic); });
+                {
+                    --scale_read_slab;          // the slab whose scales the last body read: the new tile's slab 0
+                    const uint32_t off = scale_read_offset();
+                    const uint32_t swb_at = swb + off, sab_at = sab + off;
+                    static_for<0, NF>([&](auto ic) { read_scale_at(swb_at, sab_at, ic); });
+                    ++scale_read_slab;
+                }
                 asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
                 shift_scales(I0{});
             }
