@@ -53,6 +53,7 @@ struct GemmParams {
     uint32_t groups, w_tiles;
     int out_type;
     int scale_vec;   // scale rows are 4-byte aligned: one dword load per row and slab
+    int scale_vec16; // scale rows are 16-byte aligned: one 16-byte load per row fetches the scales of four slabs
 };
 
 __device__ __forceinline__ uint32_t swz(uint32_t row, uint32_t chunk) {
@@ -903,9 +904,7 @@ int launch_tile(const GemmParams& p, int waves, uint32_t max_m_tiles, hipStream_
     const bool stream_ok = !g_disable_dl && p.scale_vec && p.kbytes % kSlabBytes == 0;
     if constexpr (TW == 256 && TM == 256 && FMT != CMX_FMT_E2M1) {
         // whole four-slab scale blocks, fetched 16 bytes per row: K a multiple of 512 bytes, 16-byte aligned scale rows
-        const bool sc16 = p.ld_as % 16 == 0 && p.ld_ws % 16 == 0 && (reinterpret_cast<uintptr_t>(p.a_scale) & 15u) == 0 &&
-                          (reinterpret_cast<uintptr_t>(p.w_scale) & 15u) == 0;
-        if ((waves == 4 || waves == 5) && stream_ok && sc16 && p.kbytes % (4 * kSlabBytes) == 0) {
+        if ((waves == 4 || waves == 5) && stream_ok && p.scale_vec16 && p.kbytes % (4 * kSlabBytes) == 0) {
             // plain bf16 output with 4-element-aligned rows takes the lean store epilogue and with it the persistent kernel
             constexpr int kLean = EPI == kEpiStore ? kEpiStoreBf16 : EPI;
             const bool lean = EPI == kEpiStore && p.out_type == CMX_OUT_BF16 && p.n % 4 == 0 && p.ldc % 4 == 0 &&
@@ -950,6 +949,11 @@ int check_operands(const void* a, uint32_t lda, const void* as, uint32_t ld_as, 
     return CMX_OK;
 }
 
+bool scales_aligned16(const void* as, uint32_t ld_as, const void* ws, uint32_t ld_ws) {
+    return ld_as % 16 == 0 && ld_ws % 16 == 0 && (reinterpret_cast<uintptr_t>(as) & 15u) == 0 &&
+           (reinterpret_cast<uintptr_t>(ws) & 15u) == 0;
+}
+
 bool scales_dword_aligned(const void* as, uint32_t ld_as, const void* ws, uint32_t ld_ws) {
     return ld_as % 4 == 0 && ld_ws % 4 == 0 && (reinterpret_cast<uintptr_t>(as) & 3u) == 0 &&
            (reinterpret_cast<uintptr_t>(ws) & 3u) == 0;
@@ -985,6 +989,7 @@ extern "C" int cmx_mx_gemm(const uint8_t* a, uint32_t lda, const uint8_t* a_scal
     p.m = m; p.n = n; p.kbytes = fmt == CMX_FMT_E2M1 ? k / 2 : k; p.kblocks = k / 32;
     p.groups = 1; p.out_type = out_type;
     p.scale_vec = scales_dword_aligned(a_scale, ld_as, b_scale, ld_bs);
+    p.scale_vec16 = scales_aligned16(a_scale, ld_as, b_scale, ld_bs);
     CMX_REQUIRE((uint64_t)n * ldb < (1ull << 32) && (uint64_t)lda * 256 < (1ull << 32), "operand tile exceeds 32-bit offsets");
     TileChoice t = choose_tile(m, n, fmt, false);
     p.w_tiles = ceil_div(n, t.tw);
@@ -1051,6 +1056,7 @@ extern "C" int cmx_mx_gmm(const uint8_t* a, uint32_t lda, const uint8_t* a_scale
     p.lda = lda; p.ld_as = ld_as; p.ldw = kbytes; p.ld_ws = k / 32; p.ldc = ldc;
     p.m = m_total; p.n = n; p.kbytes = kbytes; p.kblocks = k / 32; p.out_type = out_type;
     p.scale_vec = scales_dword_aligned(a_scale, ld_as, b_scale, k / 32);
+    p.scale_vec16 = scales_aligned16(a_scale, ld_as, b_scale, k / 32);
     return gmm_common(p, group_sizes, groups, m_total, workspace, fmt, false, static_cast<hipStream_t>(stream));
 }
 
@@ -1075,5 +1081,6 @@ extern "C" int cmx_mx_gmm_swiglu_quant(const uint8_t* a, uint32_t lda, const uin
     p.lda = lda; p.ld_as = ld_as; p.ldw = k; p.ld_ws = k / 32;
     p.m = m_total; p.n = n; p.kbytes = k; p.kblocks = k / 32; p.out_type = CMX_OUT_BF16;
     p.scale_vec = scales_dword_aligned(a_scale, ld_as, b_scale, k / 32);
+    p.scale_vec16 = scales_aligned16(a_scale, ld_as, b_scale, k / 32);
     return gmm_common(p, group_sizes, groups, m_total, workspace, CMX_FMT_E4M3, true, static_cast<hipStream_t>(stream));
 }
