@@ -30,6 +30,14 @@ __device__ __forceinline__ void static_for(F&& f) {
     }
 }
 
+// 32-bit product in one register (the compiler's own choice for "a * b + c" is the 64-bit multiply-add, whose
+// result occupies a register pair for as long as the offset lives)
+__device__ __forceinline__ uint32_t mul_lo_u32(uint32_t a, uint32_t b) {
+    uint32_t r;
+    asm("v_mul_lo_u32 %0, %1, %2" : "=v"(r) : "v"(a), "v"(b));
+    return r;
+}
+
 template <int OFF>
 __device__ __forceinline__ v4i lds_read_b128(uint32_t addr) {
     v4i r;
@@ -203,7 +211,7 @@ __global__ __launch_bounds__(256) void mx_gemm_pipe_kernel(const GemmParams p) {
         for (int i = 0; i < kTileLoads; ++i) {
             const uint32_t cr = (NW * i + wave) * 8 + (lane >> 3);
             const uint32_t logical = swz(cr, lane & 7u);
-            goff[i] = (i < kWTileLoads ? wrow_of(cr) * p.ldw : arow_of(cr - TW) * p.lda) + logical * 16;
+            goff[i] = (i < kWTileLoads ? mul_lo_u32(wrow_of(cr), p.ldw) : mul_lo_u32(arow_of(cr - TW), p.lda)) + logical * 16;
         }
         // scale dwords: this wavefront fetches those of weight rows 64*wave.. and of activation rows
         // 64*(wave mod TM/64).. (with TM = 128 two wavefronts fetch the same rows to the same place)

@@ -42,6 +42,35 @@ def test_gmm_fp8_ragged_groups(tile, counts):
     assert np.all(O.bf16_bits_to_f32(got[m:]) == 7.0)          # rows past the groups stay untouched
 
 
+@pytest.mark.parametrize("tile", [None, (256, 256, 5), (256, 128, 5), (256, 256, 8), (128, 128, 4)])
+def test_gmm_many_ragged_groups_every_row(tile):
+    """43 groups whose sizes mix empty, whole-tile and ragged cases (equal remainders included): the ragged last
+    m-tiles are numbered apart from the full ones and sorted by size, and every row must still be computed
+    exactly once with its own group's weights."""
+    from catccos_amd import ops, _lib
+    if tile:
+        _lib.load().cmx_debug_force_tile(*tile)
+    rng = np.random.default_rng(77)
+    counts = [int(c) for c in rng.integers(0, 700, size=36)] + [256, 512, 0, 128, 128, 1, 255]
+    n, k = 256, 512
+    m = sum(counts)
+    aq, asc = O.mx_quant(O.bf16_round(rng.standard_normal((m, k)).astype(np.float32)))
+    wq, ws = _weights(rng, len(counts), n, k, std=1.0)
+    c = torch.full((m, n), 7.0, dtype=torch.bfloat16, device="cuda")
+    ops.mx_gmm(dev(aq), dev(asc), dev(wq), dev(ws), dev(np.array(counts, dtype=np.int32)), k, c=c)
+    gold = O.mx_gmm_f32(aq, asc, wq, ws, counts)
+    bad, worst = close_bf16(host(c), gold)
+    assert bad == 0, (bad, worst)
+    wq, ws = _weights(rng, len(counts), n, k, std=0.06)     # gate values of order 1: SiLU stays well conditioned
+    codes, scales, act = ops.mx_gmm_swiglu_quant(dev(aq), dev(asc), dev(wq), dev(ws), dev(np.array(counts, dtype=np.int32)), k,
+                                                 want_bf16=True)
+    _, act_g, _, _ = O.gmm1_swiglu_quant(aq, asc, wq, ws, counts)
+    bad, worst = close_bf16(host(act), O.bf16_bits_to_f32(act_g), rtol=2e-2)
+    assert bad == 0, (bad, worst)
+    wq2, ws2 = O.mx_quant_bf16(host(act), "E4M3", "rne")
+    assert np.array_equal(host(scales), ws2) and np.array_equal(host(codes), wq2)
+
+
 def test_gmm_fp4_ragged_groups():
     from catccos_amd import ops
     rng = np.random.default_rng(3)
