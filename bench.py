@@ -211,7 +211,16 @@ def main() -> int:
                                  "achieved": fl2 / tg / 1e12, "peak": MXFP8_PEAK_TFLOPS, "unit": "TFLOP/s",
                                  "frac": fl2 / tg / 1e12 / MXFP8_PEAK_TFLOPS, "avg_launch_us": tg * 1e6}
         log(f"[mx_gemm cfg2] {tg*1e6:.1f} us -> {fl2/tg/1e12:.0f} TFLOP/s")
-        del a2, a2s, b2, b2s
+        # the same B stored [K, N] with scales [K/64, N, 2]: the layout pass alone (one read + one write of B)
+        bt = b2.t().contiguous()
+        bts = b2s.reshape(N2, K2 // 64, 2).permute(1, 0, 2).contiguous()
+        tl = hip_time(lambda: ops.mx_to_k_major(bt, bts, K2, N2))
+        bytes_l = 2 * (N2 * K2 + N2 * K2 // 32)
+        extra["mx_to_k_major_cfg2_B"] = {"kernel": "mx_to_k_major_kernel", "bound": "hbm", "achieved": bytes_l / tl / 1e9,
+                                         "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": bytes_l / tl / 1e9 / HBM_PEAK_GBS,
+                                         "bytes_per_launch": bytes_l, "avg_launch_us": tl * 1e6}
+        log(f"[mx_to_k_major cfg2 B] {tl*1e6:.1f} us -> {bytes_l/tl/1e9:.0f} GB/s")
+        del a2, a2s, b2, b2s, bt, bts
 
     if "fp4" in want:
         E5, T5, K5, N5 = 32, 8192, 7168, 4096

@@ -51,6 +51,7 @@ inline uint32_t scale_cols(uint32_t cols) { return round_up(ceil_div(cols, 32), 
 constexpr int kEmaxE4M3 = 8;
 constexpr int kEmaxE5M2 = 15;
 constexpr int kEmaxE2M1 = 2;
+constexpr int kEmaxE1M2 = 0;
 
 #if defined(__HIPCC__)
 
@@ -136,6 +137,23 @@ __device__ __forceinline__ uint32_t e2m1_encode(float y, bool lut) {
     return c | ((__float_as_uint(y) >> 28) & 8u);
 }
 
+// E1M2 code of |y| <= 1.75: the grid is k / 4, k = 0..7 (one exponent bit, two mantissa bits, bias 1), same
+// tie rules as E2M1.
+__device__ __forceinline__ uint32_t e1m2_encode(float y, bool lut) {
+    float a = fabsf(y);
+    uint32_t c;
+    if (lut) {
+        c = (a > 0.125f) + (a > 0.375f) + (a > 0.625f) + (a > 0.875f) + (a > 1.125f) + (a > 1.375f) + (a > 1.625f);
+        return (c != 0 && y < 0.0f) ? (c | 8u) : c;
+    }
+    c = (a > 0.125f) + (a >= 0.375f) + (a > 0.625f) + (a >= 0.875f) + (a > 1.125f) + (a >= 1.375f) + (a > 1.625f);
+    return c | ((__float_as_uint(y) >> 28) & 8u);
+}
+
+template <int FMT>
+__device__ __forceinline__ uint32_t fp4_encode(float y, bool lut) {
+    return FMT == CMX_FMT_E1M2 ? e1m2_encode(y, lut) : e2m1_encode(y, lut);
+}
 
 // ---- packed 16-bit helpers (bf16 bit patterns) and the scaled hardware casts of gfx950 ----------------
 typedef unsigned short v2u16 __attribute__((ext_vector_type(2)));

@@ -1,0 +1,220 @@
+// Layout normalisation for MX operands stored with K as the slow axis.
+//
+// The matmul kernels want both operands K-contiguous: codes [rows, K] and scales [rows, K/32].  The
+// reference's generators also write the other orientation (examples/ascend950_mxfp8_matmul_reduce_scatter/
+// scripts/gen_data_mxfp8_mmrs.py:309-330 with trans_b = 0, the setting of the fp8_mx_allgather_matmul,
+// mxfp8_matmul_alltoall and fp8_mx_alltoallv_grouped_matmul run scripts): codes [K, N] with N contiguous and
+// scales [K/64, N, 2], i.e. for every pair of K blocks the two scale bytes of a column sit together.
+// mx_to_k_major_kernel turns that into the K-contiguous form: a byte transpose of the codes and a
+// transpose of 16-bit units of the scales, both pure data movement (HBM bound: every byte is read once and
+// written once).
+//
+// One workgroup moves a 128 (K) x 128 (N) tile: dword loads along N (128-byte rows), a 4 x 4 byte transpose
+// in registers with v_perm_b32, dwords of four consecutive K bytes staged in LDS, 16-byte stores along K
+// (128-byte rows).
+#include <hip/hip_runtime.h>
+
+#include "catccos_mx.h"
+#include "mx_common.h"
+
+namespace cmx {
+namespace {
+
+constexpr int kLt = 128;                 // tile edge in bytes, both ways
+constexpr int kLtPitch = kLt / 4 + 1;    // LDS row pitch in dwords
+
+// bytes (i, j) -> (j, i) of the 4 x 4 byte matrix whose rows are r0..r3; c[j] = {r0.j, r1.j, r2.j, r3.j}
+__device__ __forceinline__ void transpose4x4(uint32_t r0, uint32_t r1, uint32_t r2, uint32_t r3, uint32_t (&c)[4]) {
+    const uint32_t t0 = __builtin_amdgcn_perm(r1, r0, 0x05010400u);   // r0.0 r1.0 r0.1 r1.1
+    const uint32_t t1 = __builtin_amdgcn_perm(r1, r0, 0x07030602u);   // r0.2 r1.2 r0.3 r1.3
+    const uint32_t t2 = __builtin_amdgcn_perm(r3, r2, 0x05010400u);
+    const uint32_t t3 = __builtin_amdgcn_perm(r3, r2, 0x07030602u);
+    c[0] = __builtin_amdgcn_perm(t2, t0, 0x05040100u);
+    c[1] = __builtin_amdgcn_perm(t2, t0, 0x07060302u);
+    c[2] = __builtin_amdgcn_perm(t3, t1, 0x05040100u);
+    c[3] = __builtin_amdgcn_perm(t3, t1, 0x07060302u);
+}
+
+// grid: (ceil(n / 128), ceil(k / 128), batch)
+__global__ __launch_bounds__(256) void mx_to_k_major_kernel(const uint8_t* __restrict__ src, uint32_t ld_src,
+                                                            const uint8_t* __restrict__ src_scale,
+                                                            uint8_t* __restrict__ dst, uint32_t ld_dst,
+                                                            uint8_t* __restrict__ dst_scale, uint32_t ld_dst_scale,
+                                                            uint32_t k, uint32_t n, uint64_t src_batch,
+                                                            uint64_t dst_batch, uint64_t src_scale_batch,
+                                                            uint64_t dst_scale_batch, int vec_in) {
+    __shared__ uint32_t tile[kLt * kLtPitch];            // [n][k / 4]
+    const uint32_t t = threadIdx.x;
+    const uint32_t n0 = blockIdx.x * kLt, k0 = blockIdx.y * kLt;
+    src += blockIdx.z * src_batch;
+    dst += blockIdx.z * dst_batch;
+    src_scale += blockIdx.z * src_scale_batch;
+    dst_scale += blockIdx.z * dst_scale_batch;
+
+    // load: thread -> column quad nq (4 bytes along N) and row quads kq, kq + 8, ...
+    const uint32_t nq = t & 31u;
+    const uint32_t ncol = n0 + 4 * nq;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const uint32_t kq = (t >> 5) + 8 * i;
+        uint32_t r[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const uint32_t kr = k0 + 4 * kq + j;
+            r[j] = 0;
+            if (kr < k) {
+                const uint8_t* p = src + (size_t)kr * ld_src + ncol;
+                if (vec_in && ncol + 4 <= n) {
+                    r[j] = *reinterpret_cast<const uint32_t*>(p);
+                } else {
+#pragma unroll
+                    for (int b = 0; b < 4; ++b)
+                        if (ncol + b < n) r[j] |= (uint32_t)p[b] << (8 * b);
+                }
+            }
+        }
+        uint32_t c[4];
+        transpose4x4(r[0], r[1], r[2], r[3], c);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) tile[(4 * nq + j) * kLtPitch + kq] = c[j];
+    }
+    __syncthreads();
+
+    // store: thread -> 16 bytes along K of row n0 + t / 8 + 32 i (k is a multiple of 64, so a piece is whole or absent)
+    const uint32_t part = t & 7u;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const uint32_t nr = (t >> 3) + 32 * i;
+        const uint32_t kc = k0 + 16 * part;
+        if (n0 + nr < n && kc < k) {
+            const uint32_t* q = tile + nr * kLtPitch + 4 * part;
+            *reinterpret_cast<uint4*>(dst + (size_t)(n0 + nr) * ld_dst + kc) = make_uint4(q[0], q[1], q[2], q[3]);
+        }
+    }
+
+    // scales: the tile spans the K-block pairs k0 / 64 and k0 / 64 + 1; [pair][n][2] -> [n][2 pair + {0, 1}]
+    if (t < (uint32_t)kLt && n0 + t < n) {
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            const uint32_t pair = k0 / 64 + h;
+            if (pair * 64 < k) {
+                const uint8_t* sp = src_scale + ((size_t)pair * n + n0 + t) * 2;
+                uint8_t* dp = dst_scale + (size_t)(n0 + t) * ld_dst_scale + 2 * pair;
+                dp[0] = sp[0];
+                dp[1] = sp[1];
+            }
+        }
+    }
+}
+
+int to_k_major(const uint8_t* src, uint32_t ld_src, const uint8_t* src_scale, uint8_t* dst, uint32_t ld_dst,
+               uint8_t* dst_scale, uint32_t ld_dst_scale, uint32_t k, uint32_t n, uint32_t batch, hipStream_t s) {
+    CMX_REQUIRE(src && src_scale && dst && dst_scale, "null pointer");
+    CMX_REQUIRE(k > 0 && k % 64 == 0, "k must be a positive multiple of 64 (scale bytes come in pairs of K blocks)");
+    CMX_REQUIRE(ld_src >= n && ld_dst >= k && ld_dst_scale >= k / 32, "row pitch smaller than a row");
+    CMX_REQUIRE(ld_dst % 16 == 0 && aligned16(dst), "destination rows must be 16-byte aligned");
+    if (n == 0 || batch == 0) return CMX_OK;
+    CMX_REQUIRE(batch <= 65535u && ceil_div(k, kLt) <= 65535u, "too many tiles for one launch");
+    const int vec_in = ld_src % 4 == 0 && (reinterpret_cast<uintptr_t>(src) & 3u) == 0;
+    dim3 grid(ceil_div(n, kLt), ceil_div(k, kLt), batch);
+    hipLaunchKernelGGL(mx_to_k_major_kernel, grid, dim3(256), 0, s, src, ld_src, src_scale, dst, ld_dst, dst_scale,
+                       ld_dst_scale, k, n, (uint64_t)k * ld_src, (uint64_t)n * ld_dst, (uint64_t)(k / 32) * n,
+                       (uint64_t)n * ld_dst_scale, vec_in);
+    CMX_LAUNCH_CHECK();
+    return CMX_OK;
+}
+
+// workspace carve-up of the *_ex entry points: normalised A (when stored [K, M]) then normalised B (when stored [K, N])
+struct ExLayout {
+    size_t a_codes, a_scales, b_codes, b_scales, total;
+};
+
+ExLayout ex_layout(uint64_t a_rows, uint64_t b_rows, uint32_t k, int trans_a, int b_k_major) {
+    ExLayout L{};
+    size_t off = 0;
+    auto take = [&](size_t bytes) {
+        const size_t at = off;
+        off += round_up_sz(bytes, 256);
+        return at;
+    };
+    if (trans_a) {
+        L.a_codes = take(a_rows * k);
+        L.a_scales = take(a_rows * (k / 32));
+    }
+    if (!b_k_major) {
+        L.b_codes = take(b_rows * k);
+        L.b_scales = take(b_rows * (k / 32));
+    }
+    L.total = off;
+    return L;
+}
+
+bool fmt_is_8bit(int fmt) { return fmt == CMX_FMT_E4M3 || fmt == CMX_FMT_E5M2; }
+
+}  // namespace
+}  // namespace cmx
+
+extern "C" int cmx_mx_to_k_major(const uint8_t* src, uint32_t ld_src, const uint8_t* src_scale, uint8_t* dst,
+                                 uint32_t ld_dst, uint8_t* dst_scale, uint32_t ld_dst_scale, uint32_t k, uint32_t n,
+                                 uint32_t batch, cmx_stream_t stream) {
+    return cmx::to_k_major(src, ld_src, src_scale, dst, ld_dst, dst_scale, ld_dst_scale, k, n, batch,
+                           static_cast<hipStream_t>(stream));
+}
+
+extern "C" size_t cmx_mx_gemm_ex_workspace_bytes(uint32_t m, uint32_t n, uint32_t k, int trans_a, int trans_b) {
+    return cmx::ex_layout(m, n, k, trans_a, trans_b).total;
+}
+
+extern "C" int cmx_mx_gemm_ex(const uint8_t* a, const uint8_t* a_scale, const uint8_t* b, const uint8_t* b_scale, void* c,
+                              uint32_t ldc, uint32_t m, uint32_t n, uint32_t k, int fmt, int out_type, int trans_a,
+                              int trans_b, void* workspace, cmx_stream_t stream) {
+    using namespace cmx;
+    if (m == 0 || n == 0) return CMX_OK;
+    CMX_REQUIRE(fmt_is_8bit(fmt), "layout normalisation covers the 8-bit element formats");
+    CMX_REQUIRE(k > 0 && k % 64 == 0, "k must be a positive multiple of 64");
+    const ExLayout L = ex_layout(m, n, k, trans_a, trans_b);
+    CMX_REQUIRE(L.total == 0 || (workspace && (reinterpret_cast<uintptr_t>(workspace) & 255u) == 0),
+                "workspace missing or not 256-byte aligned");
+    uint8_t* ws = static_cast<uint8_t*>(workspace);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (trans_a) {
+        int rc = to_k_major(a, m, a_scale, ws + L.a_codes, k, ws + L.a_scales, k / 32, k, m, 1, s);
+        if (rc != CMX_OK) return rc;
+        a = ws + L.a_codes;
+        a_scale = ws + L.a_scales;
+    }
+    if (!trans_b) {
+        int rc = to_k_major(b, n, b_scale, ws + L.b_codes, k, ws + L.b_scales, k / 32, k, n, 1, s);
+        if (rc != CMX_OK) return rc;
+        b = ws + L.b_codes;
+        b_scale = ws + L.b_scales;
+    }
+    return cmx_mx_gemm(a, k, a_scale, k / 32, b, k, b_scale, k / 32, c, ldc, m, n, k, fmt, out_type, stream);
+}
+
+extern "C" size_t cmx_mx_gmm_ex_workspace_bytes(uint32_t groups, uint32_t n, uint32_t k, int trans_b) {
+    const size_t meta = cmx::round_up_sz(cmx_mx_gmm_workspace_bytes(groups), 256);
+    return meta + cmx::ex_layout(0, (uint64_t)groups * n, k, 0, trans_b).total;
+}
+
+extern "C" int cmx_mx_gmm_ex(const uint8_t* a, const uint8_t* a_scale, const uint8_t* b, const uint8_t* b_scale, void* c,
+                             uint32_t ldc, const int32_t* group_sizes, uint32_t groups, uint32_t m_total, uint32_t n,
+                             uint32_t k, int fmt, int out_type, int trans_b, void* workspace, cmx_stream_t stream) {
+    using namespace cmx;
+    if (m_total == 0 || n == 0) return CMX_OK;
+    CMX_REQUIRE(fmt_is_8bit(fmt), "layout normalisation covers the 8-bit element formats");
+    CMX_REQUIRE(k > 0 && k % 64 == 0, "k must be a positive multiple of 64");
+    CMX_REQUIRE(groups > 0 && workspace && (reinterpret_cast<uintptr_t>(workspace) & 255u) == 0,
+                "workspace missing or not 256-byte aligned");
+    uint8_t* ws = static_cast<uint8_t*>(workspace);
+    const size_t meta = round_up_sz(cmx_mx_gmm_workspace_bytes(groups), 256);
+    if (!trans_b) {
+        const ExLayout L = ex_layout(0, (uint64_t)groups * n, k, 0, 0);
+        int rc = to_k_major(b, n, b_scale, ws + meta + L.b_codes, k, ws + meta + L.b_scales, k / 32, k, n, groups,
+                            static_cast<hipStream_t>(stream));
+        if (rc != CMX_OK) return rc;
+        b = ws + meta + L.b_codes;
+        b_scale = ws + meta + L.b_scales;
+    }
+    return cmx_mx_gmm(a, k, a_scale, k / 32, b, b_scale, c, ldc, group_sizes, groups, m_total, n, k, fmt, out_type, ws, stream);
+}

@@ -1,4 +1,4 @@
-// MX block-32 quantizer for gfx950: bf16 rows -> E4M3 / E5M2 / E2M1 codes + E8M0 scales.
+// MX block-32 quantizer for gfx950: bf16 rows -> E4M3 / E5M2 / E2M1 / E1M2 codes + E8M0 scales.
 //
 // Work split: four adjacent lanes own one 32-element block (8 bf16 = one 16-byte load each), so a
 // wavefront reads 1 KiB of contiguous input per step and every lane keeps UNROLL loads in flight.
@@ -30,8 +30,9 @@ __global__ __launch_bounds__(kThreads) void mx_quant_kernel(const uint16_t* __re
                                                             uint8_t* __restrict__ scales, uint32_t ld_scales,
                                                             uint32_t rows, uint32_t cols, uint32_t nb,
                                                             uint32_t total_blocks, int vec_in, int vec_out) {
-    constexpr int emax = FMT == CMX_FMT_E4M3 ? kEmaxE4M3 : (FMT == CMX_FMT_E5M2 ? kEmaxE5M2 : kEmaxE2M1);
-    constexpr float lim = FMT == CMX_FMT_E4M3 ? 448.0f : (FMT == CMX_FMT_E5M2 ? 57344.0f : 6.0f);
+    constexpr bool kFp4 = FMT == CMX_FMT_E2M1 || FMT == CMX_FMT_E1M2;
+    constexpr int emax = FMT == CMX_FMT_E4M3 ? kEmaxE4M3 : (FMT == CMX_FMT_E5M2 ? kEmaxE5M2 : (FMT == CMX_FMT_E2M1 ? kEmaxE2M1 : kEmaxE1M2));
+    constexpr float lim = FMT == CMX_FMT_E4M3 ? 448.0f : (FMT == CMX_FMT_E5M2 ? 57344.0f : (FMT == CMX_FMT_E2M1 ? 6.0f : 1.75f));
     const uint32_t q = threadIdx.x & 3u;
     const uint32_t b0 = blockIdx.x * (kBlocksPerIter * kUnroll) + (threadIdx.x >> 2);
 
@@ -86,10 +87,10 @@ __global__ __launch_bounds__(kThreads) void mx_quant_kernel(const uint16_t* __re
         const uint32_t row = row_[u], kb = kb_[u];
         const uint32_t col = kb * 32 + q * 8;
 
-        if constexpr (FMT == CMX_FMT_E2M1) {
+        if constexpr (kFp4) {
             uint32_t pk = 0;
 #pragma unroll
-            for (int i = 0; i < 8; ++i) pk |= e2m1_encode(y[i], LUT) << (4 * i);
+            for (int i = 0; i < 8; ++i) pk |= fp4_encode<FMT>(y[i], LUT) << (4 * i);
             uint8_t* o = codes + (size_t)row * ld_codes + (col >> 1);
             if (vec_out) {
                 if (col < cols) *reinterpret_cast<uint32_t*>(o) = pk;
@@ -210,11 +211,11 @@ __global__ void mx_dequant_kernel(const uint8_t* __restrict__ codes, uint32_t ld
     if (col >= cols || row >= rows) return;
     int e = (int)scales[(size_t)row * ld_scales + (col >> 5)] - 127;
     float v;
-    if (fmt == CMX_FMT_E2M1) {
+    if (fmt == CMX_FMT_E2M1 || fmt == CMX_FMT_E1M2) {
         uint32_t byte = codes[(size_t)row * ld_codes + (col >> 1)];
         uint32_t c = (col & 1u) ? (byte >> 4) : (byte & 0xFu);
         const float tab[8] = {0.f, 0.5f, 1.f, 1.5f, 2.f, 3.f, 4.f, 6.f};
-        v = tab[c & 7u];
+        v = fmt == CMX_FMT_E2M1 ? tab[c & 7u] : 0.25f * (float)(c & 7u);
         if (c & 8u) v = -v;
     } else {
         uint32_t c = codes[(size_t)row * ld_codes + col];
@@ -252,11 +253,12 @@ extern "C" int cmx_mx_quant(const void* x, uint32_t ld_x, uint8_t* codes, uint32
                             cmx_stream_t stream) {
     using namespace cmx;
     CMX_REQUIRE(x && codes && scales, "null pointer");
-    CMX_REQUIRE(fmt == CMX_FMT_E4M3 || fmt == CMX_FMT_E5M2 || fmt == CMX_FMT_E2M1, "unknown element format");
+    CMX_REQUIRE(fmt == CMX_FMT_E4M3 || fmt == CMX_FMT_E5M2 || fmt == CMX_FMT_E2M1 || fmt == CMX_FMT_E1M2, "unknown element format");
     CMX_REQUIRE(round_mode == CMX_ROUND_RNE || round_mode == CMX_ROUND_LUT, "unknown rounding mode");
     if (rows == 0 || cols == 0) return CMX_OK;
     const uint32_t nb = ceil_div(cols, 32);
-    const uint32_t code_cols = fmt == CMX_FMT_E2M1 ? ceil_div(cols, 2) : cols;
+    const bool fp4 = fmt == CMX_FMT_E2M1 || fmt == CMX_FMT_E1M2;
+    const uint32_t code_cols = fp4 ? ceil_div(cols, 2) : cols;
     CMX_REQUIRE(ld_x >= cols && ld_codes >= code_cols && ld_scales >= scale_cols(cols), "row pitch smaller than row");
     CMX_REQUIRE((uint64_t)rows * nb < (1ull << 32), "too many blocks for one launch");
     const uint32_t total = rows * nb;
@@ -266,7 +268,7 @@ extern "C" int cmx_mx_quant(const void* x, uint32_t ld_x, uint8_t* codes, uint32
     hipStream_t s = static_cast<hipStream_t>(stream);
     const uint16_t* xp = static_cast<const uint16_t*>(x);
     const bool lut = round_mode == CMX_ROUND_LUT;
-    const bool fast = !lut && fmt != CMX_FMT_E2M1 && cols % 32 == 0 && vec_in && vec_out &&
+    const bool fast = !lut && !fp4 && cols % 32 == 0 && vec_in && vec_out &&
                       (uint64_t)ld_x * 2 < (1ull << 32) && ceil_div(rows, kFastRows) <= 65535u;
     if (fast) {
         dim3 fgrid(ceil_div(nb, kBlocksPerIter), ceil_div(rows, kFastRows));
@@ -287,8 +289,11 @@ extern "C" int cmx_mx_quant(const void* x, uint32_t ld_x, uint8_t* codes, uint32
         case CMX_FMT_E5M2:
             return launch_quant<CMX_FMT_E5M2>(lut, grid, s, xp, ld_x, codes, ld_codes, scales, ld_scales, rows, cols, nb,
                                               total, vec_in, vec_out);
-        default:
+        case CMX_FMT_E2M1:
             return launch_quant<CMX_FMT_E2M1>(lut, grid, s, xp, ld_x, codes, ld_codes, scales, ld_scales, rows, cols, nb,
+                                              total, vec_in, vec_out);
+        default:
+            return launch_quant<CMX_FMT_E1M2>(lut, grid, s, xp, ld_x, codes, ld_codes, scales, ld_scales, rows, cols, nb,
                                               total, vec_in, vec_out);
     }
 }
@@ -298,7 +303,7 @@ extern "C" int cmx_mx_dequant(const uint8_t* codes, uint32_t ld_codes, const uin
                               cmx_stream_t stream) {
     using namespace cmx;
     CMX_REQUIRE(codes && scales && out, "null pointer");
-    CMX_REQUIRE(fmt == CMX_FMT_E4M3 || fmt == CMX_FMT_E5M2 || fmt == CMX_FMT_E2M1, "unknown element format");
+    CMX_REQUIRE(fmt == CMX_FMT_E4M3 || fmt == CMX_FMT_E5M2 || fmt == CMX_FMT_E2M1 || fmt == CMX_FMT_E1M2, "unknown element format");
     if (rows == 0 || cols == 0) return CMX_OK;
     CMX_REQUIRE(ceil_div(cols, 256) <= 65535u, "too many columns for the debug dequantizer");
     dim3 grid(rows, ceil_div(cols, 256));

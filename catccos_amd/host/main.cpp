@@ -6,7 +6,9 @@
 //     --experts E   local experts (MoE operators; default 4)      --topk T     routes per token (default 4)
 //     --data DIR    directory with the operator's input .bin files; outputs are written there too
 //                   (without it inputs are defaults / zeros and nothing is written)
-//     --fmt F       e4m3 | e5m2 | e2m1 for the quantizer and the dense matmul (default e4m3)
+//     --fmt F       e4m3 | e5m2 | e2m1 | e1m2 for the quantizer, e4m3 | e5m2 for the dense matmul (default e4m3)
+//     --transa 0|1  dense matmul: A files hold [K, M] / [K/64, M, 2] when 1 (default 0)
+//     --transb 0|1  dense matmul: B files hold [K, N] / [K/64, N, 2] when 0 (default 1: [N, K])
 //     --repeats R   launches per case (default 1)               --warmup W   untimed launches (default 5)
 //     --poison      fill workspace and outputs with 0xA5 first (stale-state check)
 //     --m0 128|256  recorded in the tiling arguments (GMM1 M tile of the reference; tile choice here is automatic)
@@ -28,7 +30,7 @@ namespace {
 
 struct Options {
     std::string op;
-    uint32_t m = 0, k = 0, n = 0, experts = 4, topK = 4, repeats = 1, warmup = 5, m0 = M0;
+    uint32_t m = 0, k = 0, n = 0, experts = 4, topK = 4, repeats = 1, warmup = 5, m0 = M0, transA = 0, transB = 1;
     std::string data, fmt = "e4m3";
     bool poison = false;
 };
@@ -47,7 +49,7 @@ Options Parse(int argc, char** argv)
 {
     if (argc < 5) {
         throw std::runtime_error("Usage: catccos_mx_run <operator> M K N [--experts E] [--topk T] [--data DIR] [--fmt F] "
-                                 "[--repeats R] [--warmup W] [--poison] [--m0 128|256]");
+                                 "[--repeats R] [--warmup W] [--poison] [--m0 128|256] [--transa 0|1] [--transb 0|1]");
     }
     Options o;
     o.op = argv[1];
@@ -65,6 +67,8 @@ Options Parse(int argc, char** argv)
         else if (a == "--repeats") o.repeats = ParsePositive(next("--repeats"), "repeats");
         else if (a == "--warmup") o.warmup = static_cast<uint32_t>(std::strtoul(next("--warmup"), nullptr, 10));
         else if (a == "--m0") o.m0 = ParsePositive(next("--m0"), "m0");
+        else if (a == "--transa") o.transA = static_cast<uint32_t>(std::strtoul(next("--transa"), nullptr, 10));
+        else if (a == "--transb") o.transB = static_cast<uint32_t>(std::strtoul(next("--transb"), nullptr, 10));
         else if (a == "--data") o.data = next("--data");
         else if (a == "--fmt") o.fmt = next("--fmt");
         else if (a == "--poison") o.poison = true;
@@ -79,6 +83,7 @@ int FormatOf(const std::string& f)
     if (f == "e4m3") return CMX_FMT_E4M3;
     if (f == "e5m2") return CMX_FMT_E5M2;
     if (f == "e2m1") return CMX_FMT_E2M1;
+    if (f == "e1m2") return CMX_FMT_E1M2;
     throw std::runtime_error("unknown element format " + f);
 }
 
@@ -101,16 +106,17 @@ int Run(int argc, char** argv)
     }
     const int fmt = FormatOf(o.fmt);
     MxQuantAllGatherOperator::ElementFormat() = fmt;
-    MxQuantAllGatherOperator::RoundMode() = fmt == CMX_FMT_E2M1 ? CMX_ROUND_LUT : CMX_ROUND_RNE;
-    Ascend950MxFp8MatmulReduceScatterOperator::ElementFormat() = fmt == CMX_FMT_E2M1 ? CMX_FMT_E4M3 : fmt;
+    const bool fp4 = fmt == CMX_FMT_E2M1 || fmt == CMX_FMT_E1M2;
+    MxQuantAllGatherOperator::RoundMode() = fp4 ? CMX_ROUND_LUT : CMX_ROUND_RNE;
+    Ascend950MxFp8MatmulReduceScatterOperator::ElementFormat() = fp4 ? CMX_FMT_E4M3 : fmt;
 
     const uint32_t rankSize = 1, rankId = 0;
     CocTilingParams tiling{};
     tiling.m = o.m;
     tiling.k = o.k;
     tiling.n = o.n;
-    tiling.transA = 0;
-    tiling.transB = 1;
+    tiling.transA = o.transA;
+    tiling.transB = o.transB;
     tiling.m0 = o.m0;
     tiling.n0 = N0;
     tiling.k0 = K0;

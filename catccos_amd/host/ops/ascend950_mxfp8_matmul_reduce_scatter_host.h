@@ -1,7 +1,10 @@
 // "Ascend950MxFp8MatmulReduceScatter" on one GPU: the device's full M x N x K MXFP8 product in bf16 (with
 // one rank the reduce-scatter is the identity).  Host contract follows
 // examples/ascend950_mxfp8_matmul_reduce_scatter/ascend950_mxfp8_matmul_reduce_scatter_host.h:28-147.
-// B must be stored transposed ([N, K] codes, [N, K/64, 2] scales; transB = 1): both operands K-contiguous.
+// Operand files come in either orientation, as the reference's generator writes them (scripts/
+// gen_data_mxfp8_mmrs.py:309-330): A [M, K] with scales [M, K/64, 2], or [K, M] with [K/64, M, 2] when
+// transA = 1; B [N, K] with [N, K/64, 2] when transB = 1 (the example's own setting), or [K, N] with
+// [K/64, N, 2] when transB = 0.  Operands that are not K-contiguous are rewritten in the workspace first.
 #ifndef ASCEND950_MXFP8_MATMUL_REDUCE_SCATTER_HOST_H
 #define ASCEND950_MXFP8_MATMUL_REDUCE_SCATTER_HOST_H
 
@@ -36,7 +39,10 @@ public:
         mxops::DeviceBufferToFile(params.ptrC, cBytes, dataFile + "/output.bin", rankId * cBytes);   // rank r at byte r*size
     }
 
-    size_t GetWorkspaceSize(const CocTilingParams&) override { return 0; }
+    size_t GetWorkspaceSize(const CocTilingParams& t) override
+    {
+        return cmx_mx_gemm_ex_workspace_bytes(t.m, t.n, t.k, static_cast<int>(t.transA), static_cast<int>(t.transB));
+    }
     CocCommType GetActualKernelType(const CocTilingParams&) override { return CocCommType::ASCEND950_MXFP8_MATMUL_REDUCE_SCATTER; }
 
     bool CheckCocTilingParams(uint32_t rankSize, const CocTilingParams& t) override
@@ -45,18 +51,18 @@ public:
             std::cerr << "Ascend950MxFp8MatmulReduceScatter: this build computes one device's product (rankSize 1)" << std::endl;
             return false;
         }
-        if (t.transA != 0 || t.transB != 1) {
-            std::cerr << "Ascend950MxFp8MatmulReduceScatter: A row-major and B transposed ([N,K]) are required" << std::endl;
+        if (t.transA > 1 || t.transB > 1) {
+            std::cerr << "Ascend950MxFp8MatmulReduceScatter: transA and transB are 0 or 1" << std::endl;
             return false;
         }
         return t.k % 64 == 0;
     }
 
-    static int Launch(void* stream, const KernelParams& params, const CocTilingParams& t)
+    static int Launch(void* stream, const KernelParams& params, uint8_t* workspace, const CocTilingParams& t)
     {
-        const uint32_t ldScale = static_cast<uint32_t>(ScaleRowBytes(t.k));
-        return cmx_mx_gemm(params.ptrA, t.k, params.customPtrs[0], ldScale, params.ptrB, t.k, params.customPtrs[1], ldScale,
-                           params.ptrC, t.n, t.m, t.n, t.k, ElementFormat(), CMX_OUT_BF16, stream);
+        return cmx_mx_gemm_ex(params.ptrA, params.customPtrs[0], params.ptrB, params.customPtrs[1], params.ptrC, t.n, t.m, t.n,
+                              t.k, ElementFormat(), CMX_OUT_BF16, static_cast<int>(t.transA), static_cast<int>(t.transB),
+                              workspace, stream);
     }
 };
 

@@ -13,13 +13,12 @@ void LaunchQuant(void* stream, uint32_t, uint64_t, KernelParams& p, uint8_t*, ui
 {
     LaunchStatus() = MxQuantAllGatherOperator::Launch(stream, p, t, 0);
 }
-void LaunchMmrs(void* stream, uint32_t, uint64_t, KernelParams& p, uint8_t*, uint8_t*, CocTilingParams& t, uint32_t transA, uint32_t transB)
+void LaunchMmrs(void* stream, uint32_t, uint64_t, KernelParams& p, uint8_t* ws, uint8_t*, CocTilingParams& t, uint32_t transA, uint32_t transB)
 {
-    if (transA != 0 || transB != 1) {
-        LaunchStatus() = CMX_EINVAL;
-        return;
-    }
-    LaunchStatus() = Ascend950MxFp8MatmulReduceScatterOperator::Launch(stream, p, t);
+    CocTilingParams tt = t;
+    tt.transA = transA;
+    tt.transB = transB;
+    LaunchStatus() = Ascend950MxFp8MatmulReduceScatterOperator::Launch(stream, p, ws, tt);
 }
 void LaunchFfn(void* stream, uint32_t, uint64_t, KernelParams& p, uint8_t* ws, uint8_t* symm, CocTilingParams& t, uint32_t, uint32_t)
 {

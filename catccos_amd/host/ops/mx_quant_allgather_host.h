@@ -11,10 +11,10 @@ class MxQuantAllGatherOperator : public CatccosOperator {
 public:
     static constexpr uint32_t MX_BLOCK_SIZE = 32;
 
-    // CMX_FMT_E4M3 (default) / CMX_FMT_E5M2 / CMX_FMT_E2M1 and CMX_ROUND_RNE / CMX_ROUND_LUT for all instances
+    // CMX_FMT_E4M3 (default) / CMX_FMT_E5M2 / CMX_FMT_E2M1 / CMX_FMT_E1M2 and CMX_ROUND_RNE / CMX_ROUND_LUT for all instances
     static int& ElementFormat() { static int fmt = CMX_FMT_E4M3; return fmt; }
     static int& RoundMode() { static int mode = CMX_ROUND_RNE; return mode; }
-    static uint32_t PackRatio() { return ElementFormat() == CMX_FMT_E2M1 ? 2 : 1; }
+    static uint32_t PackRatio() { return ElementFormat() == CMX_FMT_E2M1 || ElementFormat() == CMX_FMT_E1M2 ? 2 : 1; }
 
     static bool CheckProblemShape(uint32_t rankSize, const CocTilingParams& t)
     {

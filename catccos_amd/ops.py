@@ -11,7 +11,8 @@ import torch
 
 from . import _lib
 
-FMT = {"E4M3": 0, "E5M2": 1, "E2M1": 2}
+FMT = {"E4M3": 0, "E5M2": 1, "E2M1": 2, "E1M2": 3}
+_FP4 = ("E2M1", "E1M2")
 ROUND = {"rne": 0, "lut": 1}
 OUT = {"bf16": 0, "fp16": 1, "fp32": 2}
 _OUT_DTYPE = {"bf16": torch.bfloat16, "fp16": torch.float16, "fp32": torch.float32}
@@ -42,8 +43,8 @@ def mx_quant(x: torch.Tensor, fmt: str = "E4M3", mode: str | None = None):
     assert x.dim() == 2 and x.element_size() == 2 and x.stride(1) == 1
     rows, cols = x.shape
     if mode is None:
-        mode = "lut" if fmt == "E2M1" else "rne"
-    ccols = (cols + 1) // 2 if fmt == "E2M1" else cols
+        mode = "lut" if fmt in _FP4 else "rne"
+    ccols = (cols + 1) // 2 if fmt in _FP4 else cols
     codes = torch.empty((rows, ccols), dtype=torch.uint8, device=x.device)
     scales = torch.empty((rows, scale_cols(cols)), dtype=torch.uint8, device=x.device)
     lib = _lib.load()
@@ -70,6 +71,48 @@ def mx_gemm(a, a_scale, b, b_scale, k: int, fmt: str = "E4M3", out: str = "bf16"
     lib = _lib.load()
     _lib.check(lib.cmx_mx_gemm(_p(a), a.stride(0), _p(a_scale), a_scale.stride(0), _p(b), b.stride(0), _p(b_scale),
                                b_scale.stride(0), _p(c), n, m, n, k, FMT[fmt], OUT[out], _stream()))
+    return c
+
+
+def mx_to_k_major(src, src_scale, k: int, n: int):
+    """codes [batch, k, n] (or [k, n]) with scales [batch, k/64, n, 2] -> K-contiguous codes [batch, n, k], scales [batch, n, k/32]."""
+    _need_cuda(src, src_scale)
+    assert src.is_contiguous() and src_scale.is_contiguous()
+    batch = src.shape[0] if src.dim() == 3 else 1
+    shape = (batch, n) if src.dim() == 3 else (n,)
+    dst = torch.empty(shape + (k,), dtype=torch.uint8, device=src.device)
+    dst_scale = torch.empty(shape + (k // 32,), dtype=torch.uint8, device=src.device)
+    lib = _lib.load()
+    _lib.check(lib.cmx_mx_to_k_major(_p(src), n, _p(src_scale), _p(dst), k, _p(dst_scale), k // 32, k, n, batch, _stream()))
+    return dst, dst_scale
+
+
+def mx_gemm_ex(a, a_scale, b, b_scale, m: int, n: int, k: int, fmt: str = "E4M3", out: str = "bf16", trans_a: int = 0,
+               trans_b: int = 1) -> torch.Tensor:
+    """Dense operands in the reference's file layouts: a [m, k] (trans_a = 1: [k, m], scales [k/64, m, 2]);
+    b [n, k] (trans_b = 0: [k, n], scales [k/64, n, 2])."""
+    _need_cuda(a, a_scale, b, b_scale)
+    assert all(t.is_contiguous() for t in (a, a_scale, b, b_scale))
+    lib = _lib.load()
+    need = lib.cmx_mx_gemm_ex_workspace_bytes(m, n, k, trans_a, trans_b)
+    ws = torch.empty(max(need, 1), dtype=torch.uint8, device=a.device)
+    c = torch.empty((m, n), dtype=_OUT_DTYPE[out], device=a.device)
+    _lib.check(lib.cmx_mx_gemm_ex(_p(a), _p(a_scale), _p(b), _p(b_scale), _p(c), n, m, n, k, FMT[fmt], OUT[out], trans_a,
+                                  trans_b, _p(ws), _stream()))
+    return c
+
+
+def mx_gmm_ex(a, a_scale, b, b_scale, group_sizes, n: int, k: int, fmt: str = "E4M3", out: str = "bf16",
+              trans_b: int = 1) -> torch.Tensor:
+    """Grouped form: b [G, n, k] (trans_b = 0: [G, k, n], scales [G, k/64, n, 2])."""
+    _need_cuda(a, a_scale, b, b_scale, group_sizes)
+    assert all(t.is_contiguous() for t in (a, a_scale, b, b_scale)) and group_sizes.dtype == torch.int32
+    m, g = a.shape[0], b.shape[0]
+    lib = _lib.load()
+    ws = torch.empty(lib.cmx_mx_gmm_ex_workspace_bytes(g, n, k, trans_b), dtype=torch.uint8, device=a.device)
+    c = torch.zeros((m, n), dtype=_OUT_DTYPE[out], device=a.device)
+    _lib.check(lib.cmx_mx_gmm_ex(_p(a), _p(a_scale), _p(b), _p(b_scale), _p(c), n, _p(group_sizes), g, m, n, k, FMT[fmt],
+                                 OUT[out], trans_b, _p(ws), _stream()))
     return c
 
 

@@ -29,6 +29,7 @@ extern "C" {
 #define CMX_FMT_E4M3 0
 #define CMX_FMT_E5M2 1
 #define CMX_FMT_E2M1 2 /* FP4, two codes per byte, even column in the low nibble */
+#define CMX_FMT_E1M2 3 /* FP4 with values k/4, k = 0..7 (quantizer and dequantizer only), packed like E2M1 */
 
 /* rounding of the element cast */
 #define CMX_ROUND_RNE 0 /* IEEE nearest-even: runtime activations            */
@@ -138,6 +139,37 @@ int cmx_mx_gmm_swiglu_quant(const uint8_t* a, uint32_t lda, const uint8_t* a_sca
                             uint8_t* act_scales, uint32_t ld_acts, void* act_bf16, const int32_t* group_sizes,
                             uint32_t groups, uint32_t m_total, uint32_t n, uint32_t k, void* workspace,
                             cmx_stream_t stream);
+
+/* ------------------------------------------------------------------------------------------
+ * Operands stored with K as the slow axis.
+ * The reference's generators write B either transposed ([N, K], what cmx_mx_gemm takes) or as
+ * [K, N] codes with scales [K/64, N, 2] (examples/ascend950_mxfp8_matmul_reduce_scatter/scripts/
+ * gen_data_mxfp8_mmrs.py:309-330, trans_b = 0: the setting of examples/ascend950_fp8_mx_allgather_matmul,
+ * ascend950_mxfp8_matmul_alltoall and ascend950_fp8_mx_alltoallv_grouped_matmul scripts/run.sh:17); A with
+ * trans_a = 1 is [K, M] with scales [K/64, M, 2] (:318-321).  On the device these are the RowMajor /
+ * ColumnMajor layout tags handed to BlockMmadTla (examples/ascend950_mxfp8_matmul_reduce_scatter/main.cpp:27-32).
+ *
+ * cmx_mx_to_k_major rewrites `batch` such operands (codes [batch, k, n] with row pitch ld_src, scales
+ * [batch, k/64, n, 2] dense) as K-contiguous ones (codes [batch, n, k] with row pitch ld_dst, scales
+ * [batch, n, k/32] with row pitch ld_dst_scale).  8-bit element formats; k a multiple of 64.
+ *
+ * cmx_mx_gemm_ex / cmx_mx_gmm_ex are cmx_mx_gemm / cmx_mx_gmm for dense operands in either orientation
+ * (trans_a = 1: A is [K, M]; trans_b = 0: B is [K, N] resp. [groups, K, N]); operands that are not K-contiguous
+ * are normalised into the workspace first (one extra read and write of that operand).  The workspace
+ * must be 256-byte aligned and hold *_ex_workspace_bytes bytes (for the grouped form this includes the
+ * tile schedule metadata of cmx_mx_gmm).
+ * ---------------------------------------------------------------------------------------- */
+int cmx_mx_to_k_major(const uint8_t* src, uint32_t ld_src, const uint8_t* src_scale, uint8_t* dst, uint32_t ld_dst,
+                      uint8_t* dst_scale, uint32_t ld_dst_scale, uint32_t k, uint32_t n, uint32_t batch,
+                      cmx_stream_t stream);
+size_t cmx_mx_gemm_ex_workspace_bytes(uint32_t m, uint32_t n, uint32_t k, int trans_a, int trans_b);
+int cmx_mx_gemm_ex(const uint8_t* a, const uint8_t* a_scale, const uint8_t* b, const uint8_t* b_scale, void* c,
+                   uint32_t ldc, uint32_t m, uint32_t n, uint32_t k, int fmt, int out_type, int trans_a, int trans_b,
+                   void* workspace, cmx_stream_t stream);
+size_t cmx_mx_gmm_ex_workspace_bytes(uint32_t groups, uint32_t n, uint32_t k, int trans_b);
+int cmx_mx_gmm_ex(const uint8_t* a, const uint8_t* a_scale, const uint8_t* b, const uint8_t* b_scale, void* c,
+                  uint32_t ldc, const int32_t* group_sizes, uint32_t groups, uint32_t m_total, uint32_t n, uint32_t k,
+                  int fmt, int out_type, int trans_b, void* workspace, cmx_stream_t stream);
 
 /* ------------------------------------------------------------------------------------------
  * MoE routing: stable sort of (expert, row) pairs.

@@ -362,6 +362,32 @@ def mx_gemm_f32(a_codes, a_scales, b_codes, b_scales, fmt_a="E4M3", fmt_b="E4M3"
     return a @ b.T
 
 
+def to_file_layout(codes, scales, trans: bool):
+    """K-contiguous operand (codes [R, K], scales [R, K/32]) -> the reference's file layout.
+    trans False ("stored transposed", B with trans_b = 1 / A with trans_a = 0): codes [R, K], scales
+    [R, K/64, 2] -- the same bytes.  trans True (B with trans_b = 0 / A with trans_a = 1): codes [K, R],
+    scales [K/64, R, 2].  gen_data_mxfp8_mmrs.py:311-330 (reshape to pairs, then permute(0, 2, 1) resp.
+    permute(1, 0, 2))."""
+    codes = np.asarray(codes)
+    scales = np.asarray(scales)
+    r, k = codes.shape
+    pairs = scales[:, :k // 32].reshape(r, k // 64, 2)
+    if not trans:
+        return np.ascontiguousarray(codes), np.ascontiguousarray(pairs)
+    return np.ascontiguousarray(codes.T), np.ascontiguousarray(pairs.transpose(1, 0, 2))
+
+
+def from_file_layout(codes, scales, trans: bool):
+    """Inverse of :func:`to_file_layout`: back to codes [R, K], scales [R, K/32]."""
+    codes = np.asarray(codes)
+    scales = np.asarray(scales)
+    if not trans:
+        r, k = codes.shape
+        return np.ascontiguousarray(codes), np.ascontiguousarray(scales.reshape(r, k // 32))
+    k, r = codes.shape
+    return np.ascontiguousarray(codes.T), np.ascontiguousarray(scales.reshape(k // 64, r, 2).transpose(1, 0, 2).reshape(r, k // 32))
+
+
 def mx_gemm_bf16(*args, **kw) -> np.ndarray:
     """bf16 result (bit pattern) of :func:`mx_gemm_f32` (gen_data_moe.py:650)."""
     return f32_to_bf16_bits(mx_gemm_f32(*args, **kw))

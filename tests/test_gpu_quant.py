@@ -9,14 +9,15 @@ from tests.gpu_util import dev, host, bf16_dev
 
 pytestmark = pytest.mark.gpu
 
-CASES = [("E4M3", "rne"), ("E4M3", "lut"), ("E5M2", "rne"), ("E5M2", "lut"), ("E2M1", "lut"), ("E2M1", "rne")]
+CASES = [("E4M3", "rne"), ("E4M3", "lut"), ("E5M2", "rne"), ("E5M2", "lut"), ("E2M1", "lut"), ("E2M1", "rne"),
+         ("E1M2", "lut"), ("E1M2", "rne")]
 
 
 def _check(xbits, fmt, mode):
     from catccos_amd import ops
     q, s = ops.mx_quant(bf16_dev(xbits), fmt, mode)
     wq, ws = O.mx_quant_bf16(xbits, fmt, mode)
-    if fmt == "E2M1":
+    if fmt in ("E2M1", "E1M2"):
         wq = O.pack_fp4(wq)
     gq, gs = host(q), host(s)
     assert np.array_equal(gs, ws), f"scales differ at {np.argwhere(gs != ws)[:5]}"
@@ -48,7 +49,8 @@ def test_every_bf16_value_in_varied_company(fmt, mode):
 def test_exact_midpoints_and_clips(fmt, mode):
     """Every midpoint between adjacent grid values (where RNE and table rounding part ways) and
     values between the largest grid value and 2x it (clip), in blocks whose scale is 2^0."""
-    tab = {"E4M3": O.e4m3_table()[:127], "E5M2": O.e5m2_table()[:124], "E2M1": O.fp4_table()[:8]}[fmt]
+    tab = {"E4M3": O.e4m3_table()[:127], "E5M2": O.e5m2_table()[:124], "E2M1": O.fp4_table()[:8],
+           "E1M2": O.fp4_table("E1M2")[:8]}[fmt]
     top = float(tab[-1])
     mids = ((tab[:-1].astype(np.float64) + tab[1:]) / 2).astype(np.float32)
     mids = mids[O.bf16_round(mids) == mids]          # those exactly representable in bf16
@@ -69,7 +71,7 @@ def test_exact_midpoints_and_clips(fmt, mode):
 @pytest.mark.parametrize("rows,cols", [(1, 32), (3, 40), (5, 20), (7, 96), (2, 7168), (33, 1000), (4, 2050)])
 def test_ragged_shapes(rows, cols):
     xb = W.activations_with_outliers(rows, cols, seed=rows * 1000 + cols)
-    for fmt, mode in [("E4M3", "rne"), ("E2M1", "lut")]:
+    for fmt, mode in [("E4M3", "rne"), ("E2M1", "lut"), ("E1M2", "rne")]:
         _check(xb, fmt, mode)
 
 

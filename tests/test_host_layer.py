@@ -61,7 +61,7 @@ def _write(path, arr):
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("fmt,ofmt", [("e4m3", "E4M3"), ("e5m2", "E5M2"), ("e2m1", "E2M1")])
+@pytest.mark.parametrize("fmt,ofmt", [("e4m3", "E4M3"), ("e5m2", "E5M2"), ("e2m1", "E2M1"), ("e1m2", "E1M2")])
 def test_driver_quant(host_bin, tmp_path, fmt, ofmt):
     rows, cols = 96, 7168
     x = W.activations_with_outliers(rows, cols, seed=5)
@@ -69,8 +69,9 @@ def test_driver_quant(host_bin, tmp_path, fmt, ofmt):
     r = _run(host_bin, "MxQuantAllGather", rows, 1, cols, "--data", tmp_path, "--fmt", fmt, "--poison")
     assert r.returncode == 0, r.stdout + r.stderr
     assert "[TEST] input rank_size: 1 rank_id:0" in r.stdout and "[CONFIG]" in r.stdout
-    codes, scales = O.mx_quant_bf16(x, ofmt, "lut" if ofmt == "E2M1" else "rne")
-    if ofmt == "E2M1":
+    fp4 = ofmt in ("E2M1", "E1M2")
+    codes, scales = O.mx_quant_bf16(x, ofmt, "lut" if fp4 else "rne")
+    if fp4:
         codes = O.pack_fp4(codes)
     got = np.fromfile(tmp_path / "rank_0_output.bin", dtype=np.uint8).reshape(codes.shape)
     got_s = np.fromfile(tmp_path / "rank_0_mxscale.bin", dtype=np.uint8).reshape(scales.shape)
@@ -89,6 +90,27 @@ def test_driver_mxfp8_matmul(host_bin, tmp_path):
     assert r.returncode == 0, r.stdout + r.stderr
     got = np.fromfile(tmp_path / "output.bin", dtype=np.uint16).reshape(m, n)
     gold = O.mx_gemm_f32(aq, asc, bq, bsc)
+    assert np.allclose(O.bf16_bits_to_f32(got), gold, rtol=1e-2, atol=1e-2)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("trans_a,trans_b", [(0, 0), (1, 0), (1, 1)])
+def test_driver_mxfp8_matmul_operand_orientations(host_bin, tmp_path, trans_a, trans_b):
+    """Input files in the generator's other orientations (gen_data_mxfp8_mmrs.py:309-330), E5M2 as in the
+    reference example's main.cpp:20-21."""
+    m, k, n = 160, 512, 320
+    rng = np.random.default_rng(13)
+    aq, asc = O.mx_quant(O.bf16_round(rng.standard_normal((m, k)).astype(np.float32)), "E5M2", "rne")
+    bq, bsc = O.mx_quant(O.bf16_round(rng.standard_normal((n, k)).astype(np.float32) / np.sqrt(k)), "E5M2", "rne")
+    fa, fas = O.to_file_layout(aq, asc, bool(trans_a))
+    fb, fbs = O.to_file_layout(bq, bsc, not trans_b)
+    for stem, arr in (("a", fa), ("b", fb), ("a_scale", fas), ("b_scale", fbs)):
+        _write(tmp_path / f"rank_0_{stem}.bin", arr)
+    r = _run(host_bin, "a5mxfp8mmrs", m, k, n, "--data", tmp_path, "--fmt", "e5m2", "--transa", trans_a, "--transb", trans_b,
+             "--poison")
+    assert r.returncode == 0, r.stdout + r.stderr
+    got = np.fromfile(tmp_path / "output.bin", dtype=np.uint16).reshape(m, n)
+    gold = O.mx_gemm_f32(aq, asc, bq, bsc, "E5M2", "E5M2")
     assert np.allclose(O.bf16_bits_to_f32(got), gold, rtol=1e-2, atol=1e-2)
 
 

@@ -222,3 +222,32 @@ def test_ffn_end_to_end_small_is_self_consistent():
     ok, err, eb = O.verify_bf16(out, acc, k)
     assert ok and err == 0
     assert np.mean(out != O.f32_to_bf16_bits(acc)) < 0.02
+
+
+def test_file_layouts_of_operands_by_explicit_indexing():
+    """The [K, R] / [K/64, R, 2] file orientation, checked element by element with the index arithmetic of the
+    generator written out (gen_data_mxfp8_mmrs.py:314-330: scale (r, kb) lands at ((kb // 2) * R + r) * 2 + kb % 2),
+    and through the golden's own dequantisation of that orientation (:349-352: scales repeated 32 times along K)."""
+    rng = np.random.default_rng(21)
+    r, k = 5, 192
+    codes, scales = _rand_mx(rng, r, k)
+    fc, fs = O.to_file_layout(codes, scales, True)
+    assert fc.shape == (k, r) and fs.shape == (k // 64, r, 2)
+    flat = fs.reshape(-1)
+    for i in range(r):
+        for kk in range(k):
+            assert fc[kk, i] == codes[i, kk]
+            kb = kk // 32
+            assert flat[((kb // 2) * r + i) * 2 + kb % 2] == scales[i, kb]
+    # golden-style dequantisation of the [K, R] orientation: scale matrix [K/32, R] repeated along K
+    smat = np.zeros((k // 32, r), dtype=np.uint8)
+    for kb in range(k // 32):
+        smat[kb] = fs[kb // 2, :, kb % 2]
+    deq_file = O.decode(fc, "E4M3") * np.exp2(np.repeat(smat.astype(np.float64) - 127, 32, axis=0))
+    assert np.array_equal(deq_file.astype(np.float32), O.mx_dequant(codes, scales).T)
+    # stored-transposed orientation: the same bytes, and both directions invert
+    nc, ns = O.to_file_layout(codes, scales, False)
+    assert np.array_equal(nc, codes) and np.array_equal(ns.reshape(r, -1), scales[:, :k // 32])
+    for trans in (False, True):
+        c2, s2 = O.from_file_layout(*O.to_file_layout(codes, scales, trans), trans)
+        assert np.array_equal(c2, codes) and np.array_equal(s2, scales[:, :k // 32])

@@ -144,6 +144,29 @@ def test_fp4_rne_ties_to_even():
     assert np.array_equal(err, best)                              # always a nearest value
 
 
+def test_e1m2_lut_and_rne_against_the_grid_k_over_4():
+    """E1M2 values are k/4, k = 0..7 (gen_mx_quant_allgather_data.py:65-72, 352-376): the table encode is the
+    first arg-min over the 16 entries, RNE is round-half-even of 4|y| -- both checked by brute force over every
+    bf16 value up to the clip, plus the ties written out."""
+    y = np.array([0.125, 0.375, 0.625, 0.875, 1.125, 1.375, 1.625, -0.125, -0.0, -1.7, 1.75, 0.13], dtype=np.float32)
+    assert list(O.fp4_encode_lut(y, "E1M2")) == [0, 1, 2, 3, 4, 5, 6, 0, 0, 15, 7, 1]
+    assert list(O.fp4_encode_rne(y, "E1M2")) == [0, 2, 2, 4, 4, 6, 6, 8, 8, 15, 7, 1]
+    v = all_bf16_f32(1.75)
+    tab = O.fp4_table("E1M2")
+    want = np.argmin(np.abs(v[:, None] - tab[None, :]), axis=1).astype(np.uint8)
+    assert np.array_equal(O.fp4_encode_lut(v, "E1M2"), want)
+    k = np.rint(np.abs(v).astype(np.float64) * 4).astype(np.int64)        # numpy rint: half to even
+    assert np.array_equal(O.fp4_encode_rne(v, "E1M2"), (k | np.where(np.signbit(v), 8, 0)).astype(np.uint8))
+    # block exponent: emax 0, so amax in [1, 2) keeps scale 2^0 and amax 1.9 clips to 1.75
+    x = np.zeros((1, 32), dtype=np.float32)
+    x[0, :4] = [1.9, -0.3, 0.375, 1.0]
+    q, s = O.mx_quant(x, "E1M2", "lut")
+    assert s[0, 0] == 127 and q[0, :4].tolist() == [7, 9, 1, 4]
+    x[0, 0] = 4.0                                                          # floor(log2 4) - 0 = 2
+    q, s = O.mx_quant(x, "E1M2", "lut")
+    assert s[0, 0] == 129 and q[0, :4].tolist() == [4, 0, 0, 1]          # 1.0, -0.075 -> +0, 0.094 -> 0, 0.25
+
+
 def test_fp4_pack_closed_form():
     rng = np.random.default_rng(3)
     c = rng.integers(0, 16, size=(5, 64), dtype=np.uint8)
@@ -166,7 +189,8 @@ def test_mx_quant_block_known_answers():
     assert np.all(q[0, 64:] == 0) and np.all(q[1, 1:] == 0)
 
 
-@pytest.mark.parametrize("fmt,mode", [("E4M3", "rne"), ("E4M3", "lut"), ("E5M2", "rne"), ("E2M1", "lut"), ("E2M1", "rne")])
+@pytest.mark.parametrize("fmt,mode", [("E4M3", "rne"), ("E4M3", "lut"), ("E5M2", "rne"), ("E2M1", "lut"), ("E2M1", "rne"),
+                                      ("E1M2", "lut"), ("E1M2", "rne")])
 def test_mx_quant_is_idempotent_on_its_own_output(fmt, mode):
     """The reference's byte-exact protocol feeds the quantizer its own dequantized
     output re-encoded as bf16 (ascend950_mx_quant_allgather/scripts/run.sh:78-141)."""
