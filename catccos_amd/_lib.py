@@ -50,6 +50,10 @@ SIGNATURES = {
     "cmx_mx_gemm_ex": (i32, [u8p, u8p, u8p, u8p, vp, u32, u32, u32, u32, i32, i32, i32, i32, vp, vp]),
     "cmx_mx_gmm_ex_workspace_bytes": (sz, [u32, u32, u32, i32]),
     "cmx_mx_gmm_ex": (i32, [u8p, u8p, u8p, u8p, vp, u32, i32p, u32, u32, u32, u32, i32, i32, i32, vp, vp]),
+    "cmx_int8_quant_scatter": (i32, [vp, u32, i32p, vp, u32, f32p, u32, u32, u32, vp]),
+    "cmx_bytes_to_k_major": (i32, [u8p, u32, u8p, u32, u32, u32, u32, vp]),
+    "cmx_int8_gmm_workspace_bytes": (sz, [u32, u32, u32, i32]),
+    "cmx_int8_gmm_dequant_swiglu": (i32, [vp, u32, f32p, vp, f32p, u32, vp, u32, i32, i32p, u32, u32, u32, u32, i32, vp, vp]),
     "cmx_moe_routing_workspace_bytes": (sz, [u32, u32]),
     "cmx_moe_init_routing": (i32, [i32p, u32, u32, u32, i32p, i32p, i32p, vp, vp]),
     "cmx_packed_row_bytes": (u32, [u32]),

@@ -249,6 +249,56 @@ __global__ void fill_i32_kernel(int32_t* p, uint32_t n, int32_t v) {
     if (i < n) p[i] = v;
 }
 
+// ---- per-token INT8 quantise + scatter -------------------------------------------------------------
+// One workgroup per token: q = rint(x * 127 / rowmax) (round half to even), scale = rowmax / 127, the
+// row written to each of its top_k destinations.  The row is read twice (maximum, then codes); the second
+// read comes from the cache.  k % 8 == 0, rows 16-byte aligned.
+__global__ __launch_bounds__(256) void int8_quant_scatter_kernel(const uint16_t* __restrict__ x, uint32_t ld_x,
+                                                                 const int32_t* __restrict__ src2sorted,
+                                                                 int8_t* __restrict__ codes, uint32_t ld_codes,
+                                                                 float* __restrict__ scales, uint32_t k, uint32_t top_k) {
+    __shared__ uint32_t wave_max[4];
+    const uint32_t t = blockIdx.x;
+    const uint16_t* row = x + (size_t)t * ld_x;
+    const uint32_t chunks = k / 8;
+    uint32_t m = 0;                                     // largest sign-cleared bf16 pattern == largest magnitude
+    for (uint32_t c = threadIdx.x; c < chunks; c += 256) {
+        const uint4 v = *reinterpret_cast<const uint4*>(row + 8 * c);
+        m = pk_max_u16(m, v.x & 0x7FFF7FFFu);
+        m = pk_max_u16(m, v.y & 0x7FFF7FFFu);
+        m = pk_max_u16(m, v.z & 0x7FFF7FFFu);
+        m = pk_max_u16(m, v.w & 0x7FFF7FFFu);
+    }
+    m = max(m & 0xFFFFu, m >> 16);
+#pragma unroll
+    for (int d = 32; d >= 1; d >>= 1) m = max(m, (uint32_t)__shfl_xor((int)m, d));
+    if ((threadIdx.x & 63u) == 0) wave_max[threadIdx.x >> 6] = m;
+    __syncthreads();
+    m = max(max(wave_max[0], wave_max[1]), max(wave_max[2], wave_max[3]));
+    const float rowmax = __uint_as_float(m << 16);
+    const bool zero = !(rowmax > 0.0f);                 // an all-zero row: codes 0, scale 0
+    const float div = zero ? 1.0f : rowmax;
+    if (threadIdx.x < top_k) {
+        const int32_t dst = src2sorted ? src2sorted[t * top_k + threadIdx.x] : (int32_t)t;
+        if (dst >= 0) scales[dst] = __fdiv_rn(rowmax, 127.0f);
+    }
+    for (uint32_t c = threadIdx.x; c < chunks; c += 256) {
+        const uint4 v = *reinterpret_cast<const uint4*>(row + 8 * c);
+        const uint32_t d[4] = {v.x, v.y, v.z, v.w};
+        uint32_t out[2] = {0, 0};
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const float xv = __uint_as_float((i & 1) ? (d[i >> 1] & 0xFFFF0000u) : (d[i >> 1] << 16));
+            const int q = zero ? 0 : (int)rintf(__fdiv_rn(__fmul_rn(xv, 127.0f), div));
+            out[i >> 2] |= ((uint32_t)q & 0xFFu) << (8 * (i & 3));
+        }
+        for (uint32_t r = 0; r < top_k; ++r) {
+            const int32_t dst = src2sorted ? src2sorted[t * top_k + r] : (int32_t)t;
+            if (dst >= 0) *reinterpret_cast<uint2*>(codes + (size_t)dst * ld_codes + 8 * c) = make_uint2(out[0], out[1]);
+        }
+    }
+}
+
 }  // namespace
 }  // namespace cmx
 
@@ -307,6 +357,24 @@ extern "C" int cmx_quant_scatter(const void* x, uint32_t ld_x, const int32_t* sr
     hipLaunchKernelGGL(quant_scatter_kernel, dim3(ceil_div(total, 64)), dim3(256), 0, static_cast<hipStream_t>(stream),
                        static_cast<const uint16_t*>(x), ld_x, src2sorted, out_codes, ld_out, out_scales, ld_outs, tokens,
                        k, top_k, nb, total);
+    CMX_LAUNCH_CHECK();
+    return CMX_OK;
+}
+
+extern "C" int cmx_int8_quant_scatter(const void* x, uint32_t ld_x, const int32_t* src2sorted, int8_t* codes,
+                                      uint32_t ld_codes, float* scales, uint32_t tokens, uint32_t k, uint32_t top_k,
+                                      cmx_stream_t stream) {
+    using namespace cmx;
+    CMX_REQUIRE(x && codes && scales, "null pointer");
+    if (tokens == 0 || k == 0) return CMX_OK;
+    CMX_REQUIRE(top_k >= 1 && top_k <= 256, "top_k must be in [1, 256]");
+    CMX_REQUIRE(src2sorted != nullptr || top_k == 1, "without a destination table every token has one destination");
+    CMX_REQUIRE(k % 8 == 0, "k must be a multiple of 8");
+    CMX_REQUIRE(ld_x >= k && ld_x % 8 == 0 && aligned16(x), "input rows must be 16-byte aligned");
+    CMX_REQUIRE(ld_codes >= k && ld_codes % 8 == 0 && (reinterpret_cast<uintptr_t>(codes) & 7u) == 0,
+                "output rows must be 8-byte aligned");
+    hipLaunchKernelGGL(int8_quant_scatter_kernel, dim3(tokens), dim3(256), 0, static_cast<hipStream_t>(stream),
+                       static_cast<const uint16_t*>(x), ld_x, src2sorted, codes, ld_codes, scales, k, top_k);
     CMX_LAUNCH_CHECK();
     return CMX_OK;
 }

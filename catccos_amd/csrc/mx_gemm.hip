@@ -34,7 +34,11 @@ constexpr int kXcds = 8;
 
 // kEpiStoreBf16: bf16 output whose rows and row pitch are multiples of four elements (one 8-byte store per
 // accumulator quad, no per-element edge handling): small enough to sit inside a persistent kernel's tile loop
-enum Epilogue { kEpiStore = 0, kEpiSwigluQuant = 1, kEpiStoreBf16 = 2 };
+enum Epilogue { kEpiStore = 0, kEpiSwigluQuant = 1, kEpiStoreBf16 = 2, kEpiI8DequantSwiglu = 3 };
+// epilogues whose weight tile pairs gate rows (first half of N) with their up partners (second half)
+constexpr bool epi_pairs_gate_up(int epi) { return epi == kEpiSwigluQuant || epi == kEpiI8DequantSwiglu; }
+// element "format" of the INT8 path inside the kernel templates (the public format codes are the MX ones)
+constexpr int kFmtI8 = 8;
 
 struct GemmParams {
     const uint8_t* a;        // activations codes
@@ -98,6 +102,18 @@ __device__ __forceinline__ v16f mfma<CMX_FMT_E2M1>(v8i w, v8i a, v16f c, int sel
         case 2: return CMX_MFMA_CASE(4, 2);
         default: return CMX_MFMA_CASE(4, 3);
     }
+}
+
+// INT8: one 64-deep K step is two v_mfma_i32_32x32x32_i8, fed by the two halves of the same fragment registers
+// (any fixed assignment of the 32 K positions to lanes and registers gives the same integer sum, as long as both
+// operands use the same one); the INT32 accumulators travel in the fp32 accumulator type bit for bit.
+template <>
+__device__ __forceinline__ v16f mfma<kFmtI8>(v8i w, v8i a, v16f c, int, int, int) {
+    typedef int v16i __attribute__((ext_vector_type(16)));
+    v16i acc = __builtin_bit_cast(v16i, c);
+    acc = __builtin_amdgcn_mfma_i32_32x32x32_i8((v4i){w[0], w[1], w[2], w[3]}, (v4i){a[0], a[1], a[2], a[3]}, acc, 0, 0, 0);
+    acc = __builtin_amdgcn_mfma_i32_32x32x32_i8((v4i){w[4], w[5], w[6], w[7]}, (v4i){a[4], a[5], a[6], a[7]}, acc, 0, 0, 0);
+    return __builtin_bit_cast(v16f, acc);
 }
 
 // g / (1 + exp(-g)) * u with the hardware exponential and reciprocal (about 1 ulp each; the result is rounded
@@ -181,7 +197,7 @@ __device__ __forceinline__ bool locate_tile(const GemmParams& p, Tile& t) {
 // LDS/tile row of a wavefront's weight fragment f (gate fragments first, their up partners second)
 template <int TW, int WW, int EPI, int FW>
 __device__ __forceinline__ uint32_t wfrag_row_of(uint32_t ww, int f) {
-    if (EPI == kEpiSwigluQuant)
+    if (epi_pairs_gate_up(EPI))
         return f < FW / 2 ? ww * (TW / 2 / WW) + f * 32 : TW / 2 + ww * (TW / 2 / WW) + (f - FW / 2) * 32;
     return ww * (TW / WW) + f * 32;
 }
@@ -241,6 +257,68 @@ __device__ __forceinline__ void epilogue(const GemmParams& p, const Tile& tc, v1
                     } else {
                         float* o = reinterpret_cast<float*>(p.c) + mrow * p.ldc + ncol;
                         for (uint32_t i = 0; i < 4 && ncol + i < p.n; ++i) o[i] = v[i];
+                    }
+                }
+            }
+        }
+    } else if constexpr (EPI == kEpiI8DequantSwiglu) {
+        // INT32 sums -> fp32 * per-channel scale -> fp16 -> fp32 * per-token scale -> x0 * sigmoid(x0) * gate, fp32 out.
+        // w_scale holds the fp32 channel scales of all groups ([groups * n], element stride ld_ws), a_scale the fp32
+        // per-row scales.
+        typedef int v16i __attribute__((ext_vector_type(16)));
+        const uint32_t half = p.n >> 1;
+        const float* ch = reinterpret_cast<const float*>(p.w_scale) + (size_t)tc.g * p.n * p.ld_ws;
+        const float* ts = reinterpret_cast<const float*>(p.a_scale);
+        float* const out = reinterpret_cast<float*>(p.c);
+        const bool vec = p.ldc % 4 == 0 && (reinterpret_cast<uintptr_t>(p.c) & 15u) == 0;
+#pragma unroll
+        for (int f = 0; f < FW / 2; ++f) {
+            const uint32_t ncol0 = wt * (TW / 2) + ww * (TW / 2 / WW) + f * 32;
+            float cg[16], cu[16];
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const uint32_t ncol = ncol0 + 8 * (r >> 2) + 4 * lh + (r & 3);
+                const uint32_t nc = ncol < half ? ncol : half - 1;
+                cg[r] = ch[(size_t)nc * p.ld_ws];
+                cu[r] = ch[(size_t)(half + nc) * p.ld_ws];
+            }
+#pragma unroll
+            for (int fm = 0; fm < FM; ++fm) {
+                const uint32_t mloc = wm * (TM / WM) + fm * 32 + l32;
+                if (mloc >= rows_valid) continue;
+                const size_t mrow = (size_t)(row0 + mloc);
+                const float tsv = ts[mrow];
+                const v16i ig = __builtin_bit_cast(v16i, acc[f][fm]), iu = __builtin_bit_cast(v16i, acc[f + FW / 2][fm]);
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    float y[4];
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        const int r = 4 * q + i;
+                        const float x0 = __fmul_rn((float)(_Float16)__fmul_rn((float)ig[r], cg[r]), tsv);
+                        const float gate = __fmul_rn((float)(_Float16)__fmul_rn((float)iu[r], cu[r]), tsv);
+                        y[i] = __fmul_rn(__fmul_rn(x0, __builtin_amdgcn_rcpf(1.0f + __expf(-x0))), gate);
+                    }
+                    const uint32_t ncol = ncol0 + 8 * q + 4 * lh;
+                    const bool whole = vec && ncol + 4 <= half;
+                    if (p.out_type == CMX_OUT_FP32) {
+                        float* o = out + mrow * p.ldc + ncol;
+                        if (whole) {
+                            *reinterpret_cast<float4*>(o) = make_float4(y[0], y[1], y[2], y[3]);
+                        } else {
+                            for (uint32_t i = 0; i < 4 && ncol + i < half; ++i) o[i] = y[i];
+                        }
+                    } else {
+                        uint16_t h[4];
+#pragma unroll
+                        for (int i = 0; i < 4; ++i)
+                            h[i] = p.out_type == CMX_OUT_FP16 ? __builtin_bit_cast(uint16_t, (_Float16)y[i]) : (uint16_t)f32_to_bf16(y[i]);
+                        uint16_t* o = reinterpret_cast<uint16_t*>(p.c) + mrow * p.ldc + ncol;
+                        if (whole) {
+                            *reinterpret_cast<uint2*>(o) = make_uint2(h[0] | ((uint32_t)h[1] << 16), h[2] | ((uint32_t)h[3] << 16));
+                        } else {
+                            for (uint32_t i = 0; i < 4 && ncol + i < half; ++i) o[i] = h[i];
+                        }
                     }
                 }
             }
@@ -319,7 +397,7 @@ __global__ __launch_bounds__(64 * WW * WM) void mx_gemm_kernel(const GemmParams 
     constexpr int kWLoads = TW / kRowsPerPass;         // 16-byte chunks per thread per slab
     constexpr int kALoads = TM / kRowsPerPass;
     static_assert(FW >= 1 && FM >= 1 && kWLoads >= 1 && kALoads >= 1, "tile too small for the wavefront grid");
-    static_assert(EPI != kEpiSwigluQuant || (FW % 2 == 0), "gate/up fragments come in pairs");
+    static_assert(!epi_pairs_gate_up(EPI) || (FW % 2 == 0), "gate/up fragments come in pairs");
     static_assert(TW <= NT && TM <= NT, "one scale row per thread");
     constexpr int kStageBytes = (TW + TM) * kSlabBytes + (TW + TM) * 4 * kScaleDw;
 
@@ -345,7 +423,7 @@ __global__ __launch_bounds__(64 * WW * WM) void mx_gemm_kernel(const GemmParams 
     // global weight row of LDS tile row r (rows past the matrix repeat the last one; masked at the store)
     auto wrow_of = [&](uint32_t r) -> uint32_t {
         uint32_t gr;
-        if (EPI == kEpiSwigluQuant) {
+        if (epi_pairs_gate_up(EPI)) {
             const uint32_t half = p.n >> 1;
             uint32_t rr = r < TW / 2 ? wt * (TW / 2) + r : wt * (TW / 2) + (r - TW / 2);
             rr = rr < half ? rr : half - 1;
@@ -541,8 +619,10 @@ __global__ __launch_bounds__(64 * WW * WM) void mx_gemm_dl_kernel(const GemmPara
     constexpr int NW = WW * WM;                        // wavefronts: 4 (one per SIMD) or 8 (two per SIMD)
     static_assert(NW == 4 || NW == 8, "four or eight wavefronts per workgroup");
     constexpr bool kFp4 = FMT == CMX_FMT_E2M1;
+    constexpr bool kI8 = FMT == kFmtI8;                // INT8: no block scales at all
     constexpr int kSub = kFp4 ? 4 : 2;                 // MFMA steps (64 K elements each) per slab
-    constexpr int kScaleDw = kFp4 ? 2 : 1;             // scale dwords per row per slab
+    constexpr int kScaleDw = kI8 ? 0 : (kFp4 ? 2 : 1); // scale dwords per row per slab
+    constexpr int kScaleDwA = kScaleDw ? kScaleDw : 1; // array extent
     constexpr int FW = TW / WW / 32, FM = TM / WM / 32;
     constexpr int kRows = TW + TM;                     // W tile rows then A tile rows
     constexpr int kTileLoads = kRows / (8 * NW);       // direct loads per thread and slab (8 rows per wavefront-load)
@@ -554,7 +634,7 @@ __global__ __launch_bounds__(64 * WW * WM) void mx_gemm_dl_kernel(const GemmPara
     constexpr int kLoadsPerSlab = kTileLoads + kScalePerWave * kScaleDw;
     static_assert(TW % (8 * NW) == 0 && TM % (8 * NW) == 0 && TW % 64 == 0 && TM % 64 == 0, "tile shape");
     static_assert(FW >= 1 && FM >= 1, "tile too small for the wavefront grid");
-    static_assert(EPI != kEpiSwigluQuant || (FW % 2 == 0), "gate/up fragments come in pairs");
+    static_assert(!epi_pairs_gate_up(EPI) || (FW % 2 == 0), "gate/up fragments come in pairs");
 
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     uint32_t* const sScale = reinterpret_cast<uint32_t*>(smem + 2 * kSlotBytes);
@@ -578,7 +658,7 @@ __global__ __launch_bounds__(64 * WW * WM) void mx_gemm_dl_kernel(const GemmPara
 
     auto wrow_of = [&](uint32_t r) -> uint32_t {
         uint32_t gr;
-        if (EPI == kEpiSwigluQuant) {
+        if (epi_pairs_gate_up(EPI)) {
             const uint32_t half = p.n >> 1;
             uint32_t rr = r < TW / 2 ? wt * (TW / 2) + r : wt * (TW / 2) + (r - TW / 2);
             rr = rr < half ? rr : half - 1;
@@ -674,7 +754,7 @@ __global__ __launch_bounds__(64 * WW * WM) void mx_gemm_dl_kernel(const GemmPara
             for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
 
     v8i wf[2][FW], af[2][FM];
-    uint32_t sw[kScaleDw][FW], sa[kScaleDw][FM], swn[kScaleDw][FW], san[kScaleDw][FM];
+    uint32_t sw[kScaleDwA][FW] = {}, sa[kScaleDwA][FM] = {}, swn[kScaleDwA][FW] = {}, san[kScaleDwA][FM] = {};
 
     auto read_frags = [&](uint32_t slab, int h, int buf) {
         const uint8_t* st = smem + (slab & 1u) * kSlotBytes;
@@ -683,7 +763,7 @@ __global__ __launch_bounds__(64 * WW * WM) void mx_gemm_dl_kernel(const GemmPara
 #pragma unroll
         for (int f = 0; f < FW; ++f) wf[buf][f] = read_frag(st, wfrag_row(f) + l32, h);
     };
-    auto read_scales = [&](uint32_t slab, uint32_t (&w_)[kScaleDw][FW], uint32_t (&a_)[kScaleDw][FM]) {
+    auto read_scales = [&](uint32_t slab, uint32_t (&w_)[kScaleDwA][FW], uint32_t (&a_)[kScaleDwA][FM]) {
         const uint32_t* sc = sScale + (slab & 1u) * kScaleSlot;
 #pragma unroll
         for (int d = 0; d < kScaleDw; ++d) {
@@ -719,7 +799,7 @@ __global__ __launch_bounds__(64 * WW * WM) void mx_gemm_dl_kernel(const GemmPara
             // MFMA time of other instructions sits between two MFMAs: spread the LDS reads and the
             // LDS-DMA loads of this step evenly behind the MFMAs instead of clustering them.
             {
-                constexpr int kMfmas = FW * FM;
+                constexpr int kMfmas = FW * FM * (kI8 ? 2 : 1);
                 constexpr int kFragReads = (FW + FM) * (kFp4 ? 1 : 2);
                 constexpr int kDs = kFragReads + (FW + FM) * kScaleDw;     // refill step also reads the scales
                 constexpr int kDsPer = (kDs + kMfmas - 1) / kMfmas;
@@ -1060,6 +1140,61 @@ extern "C" int cmx_mx_gmm(const uint8_t* a, uint32_t lda, const uint8_t* a_scale
     p.scale_vec = scales_dword_aligned(a_scale, ld_as, b_scale, k / 32);
     p.scale_vec16 = scales_aligned16(a_scale, ld_as, b_scale, k / 32);
     return gmm_common(p, group_sizes, groups, m_total, workspace, fmt, false, static_cast<hipStream_t>(stream));
+}
+
+extern "C" size_t cmx_int8_gmm_workspace_bytes(uint32_t groups, uint32_t n, uint32_t k, int trans_b) {
+    const size_t meta = cmx::round_up_sz(cmx_mx_gmm_workspace_bytes(groups), 256);
+    return meta + (trans_b ? 0 : cmx::round_up_sz((size_t)groups * n * k, 256));
+}
+
+extern "C" int cmx_int8_gmm_dequant_swiglu(const int8_t* a, uint32_t lda, const float* token_scale, const int8_t* b,
+                                           const float* channel_scale, uint32_t channel_scale_stride, void* out,
+                                           uint32_t ld_out, int out_type, const int32_t* group_sizes, uint32_t groups,
+                                           uint32_t m_total, uint32_t n, uint32_t k, int trans_b, void* workspace,
+                                           cmx_stream_t stream) {
+    using namespace cmx;
+    if (m_total == 0 || n == 0) return CMX_OK;
+    CMX_REQUIRE(a && token_scale && b && channel_scale && out && group_sizes && workspace, "null pointer");
+    CMX_REQUIRE(groups > 0 && groups <= 65536, "bad group count");
+    CMX_REQUIRE(k > 0 && k % kSlabBytes == 0 && k < (1u << 17), "k must be a multiple of 128 below 131072 (INT32 accumulation)");
+    CMX_REQUIRE(n % 64 == 0, "n must be a multiple of 64 (32-wide gate and up fragments)");
+    CMX_REQUIRE(lda >= k && lda % 16 == 0 && aligned16(a) && aligned16(b), "operand rows must be 16-byte aligned");
+    CMX_REQUIRE(ld_out >= n / 2 && channel_scale_stride >= 1, "bad output pitch or scale stride");
+    CMX_REQUIRE(out_type == CMX_OUT_BF16 || out_type == CMX_OUT_FP16 || out_type == CMX_OUT_FP32, "unknown output type");
+    CMX_REQUIRE((reinterpret_cast<uintptr_t>(workspace) & 255u) == 0, "workspace must be 256-byte aligned");
+    CMX_REQUIRE((uint64_t)n * k < (1ull << 32) && (uint64_t)lda * 256 < (1ull << 32), "operand tile exceeds 32-bit offsets");
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    uint8_t* ws = static_cast<uint8_t*>(workspace);
+    const uint8_t* w = reinterpret_cast<const uint8_t*>(b);
+    if (!trans_b) {
+        // weights stored [groups, k, n]: rewrite them K-contiguous behind the schedule metadata
+        uint8_t* wt = ws + round_up_sz(cmx_mx_gmm_workspace_bytes(groups), 256);
+        int rc = cmx_bytes_to_k_major(w, n, wt, k, k, n, groups, stream);
+        if (rc != CMX_OK) return rc;
+        w = wt;
+    }
+    GemmParams p{};
+    p.a = reinterpret_cast<const uint8_t*>(a);
+    p.a_scale = reinterpret_cast<const uint8_t*>(token_scale);
+    p.w = w;
+    p.w_scale = reinterpret_cast<const uint8_t*>(channel_scale);
+    p.c = out;
+    p.lda = lda; p.ld_as = 0; p.ldw = k; p.ld_ws = channel_scale_stride; p.ldc = ld_out;
+    p.m = m_total; p.n = n; p.kbytes = k; p.kblocks = k / 32; p.out_type = out_type;
+    p.scale_vec = 1;
+    int32_t* row_off = reinterpret_cast<int32_t*>(ws);
+    int32_t* tile_pref = row_off + (groups + 1);
+    int32_t* tile_ctr = tile_pref + (groups + 1);
+    constexpr int kTile = 256;
+    hipLaunchKernelGGL(gmm_prepare_kernel, dim3(1), dim3(256), 0, s, group_sizes, groups, (uint32_t)kTile, row_off, tile_pref,
+                       tile_ctr);
+    CMX_LAUNCH_CHECK();
+    p.row_off = row_off;
+    p.tile_pref = tile_pref;
+    p.tile_ctr = tile_ctr;
+    p.groups = groups;
+    p.w_tiles = ceil_div(n / 2, kTile / 2);
+    return launch_gemm_dl<kFmtI8, kTile, kTile, 2, 4, kEpiI8DequantSwiglu>(p, m_total / kTile + groups, s);
 }
 
 extern "C" int cmx_mx_gmm_swiglu_quant(const uint8_t* a, uint32_t lda, const uint8_t* a_scale, uint32_t ld_as,

@@ -48,8 +48,10 @@ __global__ __launch_bounds__(256) void mx_to_k_major_kernel(const uint8_t* __res
     const uint32_t n0 = blockIdx.x * kLt, k0 = blockIdx.y * kLt;
     src += blockIdx.z * src_batch;
     dst += blockIdx.z * dst_batch;
-    src_scale += blockIdx.z * src_scale_batch;
-    dst_scale += blockIdx.z * dst_scale_batch;
+    if (src_scale != nullptr) {
+        src_scale += blockIdx.z * src_scale_batch;
+        dst_scale += blockIdx.z * dst_scale_batch;
+    }
 
     // load: thread -> column quad nq (4 bytes along N) and row quads kq, kq + 8, ...
     const uint32_t nq = t & 31u;
@@ -93,7 +95,7 @@ __global__ __launch_bounds__(256) void mx_to_k_major_kernel(const uint8_t* __res
     }
 
     // scales: the tile spans the K-block pairs k0 / 64 and k0 / 64 + 1; [pair][n][2] -> [n][2 pair + {0, 1}]
-    if (t < (uint32_t)kLt && n0 + t < n) {
+    if (src_scale != nullptr && t < (uint32_t)kLt && n0 + t < n) {
 #pragma unroll
         for (int h = 0; h < 2; ++h) {
             const uint32_t pair = k0 / 64 + h;
@@ -109,9 +111,9 @@ __global__ __launch_bounds__(256) void mx_to_k_major_kernel(const uint8_t* __res
 
 int to_k_major(const uint8_t* src, uint32_t ld_src, const uint8_t* src_scale, uint8_t* dst, uint32_t ld_dst,
                uint8_t* dst_scale, uint32_t ld_dst_scale, uint32_t k, uint32_t n, uint32_t batch, hipStream_t s) {
-    CMX_REQUIRE(src && src_scale && dst && dst_scale, "null pointer");
+    CMX_REQUIRE(src && dst && (src_scale == nullptr) == (dst_scale == nullptr), "null pointer");
     CMX_REQUIRE(k > 0 && k % 64 == 0, "k must be a positive multiple of 64 (scale bytes come in pairs of K blocks)");
-    CMX_REQUIRE(ld_src >= n && ld_dst >= k && ld_dst_scale >= k / 32, "row pitch smaller than a row");
+    CMX_REQUIRE(ld_src >= n && ld_dst >= k && (dst_scale == nullptr || ld_dst_scale >= k / 32), "row pitch smaller than a row");
     CMX_REQUIRE(ld_dst % 16 == 0 && aligned16(dst), "destination rows must be 16-byte aligned");
     if (n == 0 || batch == 0) return CMX_OK;
     CMX_REQUIRE(batch <= 65535u && ceil_div(k, kLt) <= 65535u, "too many tiles for one launch");
@@ -157,8 +159,18 @@ bool fmt_is_8bit(int fmt) { return fmt == CMX_FMT_E4M3 || fmt == CMX_FMT_E5M2; }
 extern "C" int cmx_mx_to_k_major(const uint8_t* src, uint32_t ld_src, const uint8_t* src_scale, uint8_t* dst,
                                  uint32_t ld_dst, uint8_t* dst_scale, uint32_t ld_dst_scale, uint32_t k, uint32_t n,
                                  uint32_t batch, cmx_stream_t stream) {
+    if (!src_scale || !dst_scale) {
+        cmx::set_error("null pointer");
+        return CMX_EINVAL;
+    }
     return cmx::to_k_major(src, ld_src, src_scale, dst, ld_dst, dst_scale, ld_dst_scale, k, n, batch,
                            static_cast<hipStream_t>(stream));
+}
+
+// the code part alone (INT8 weights stored [batch, k, n] -> [batch, n, k])
+extern "C" int cmx_bytes_to_k_major(const uint8_t* src, uint32_t ld_src, uint8_t* dst, uint32_t ld_dst, uint32_t k, uint32_t n,
+                                    uint32_t batch, cmx_stream_t stream) {
+    return cmx::to_k_major(src, ld_src, nullptr, dst, ld_dst, nullptr, 0, k, n, batch, static_cast<hipStream_t>(stream));
 }
 
 extern "C" size_t cmx_mx_gemm_ex_workspace_bytes(uint32_t m, uint32_t n, uint32_t k, int trans_a, int trans_b) {

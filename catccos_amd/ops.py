@@ -116,6 +116,33 @@ def mx_gmm_ex(a, a_scale, b, b_scale, group_sizes, n: int, k: int, fmt: str = "E
     return c
 
 
+def int8_quant_scatter(x: torch.Tensor, src2sorted, top_k: int = 1):
+    """x bf16 [tokens, k] -> (codes int8 [tokens*top_k, k], scales fp32 [tokens*top_k]); row t goes to src2sorted[t*top_k + r]."""
+    _need_cuda(x, src2sorted)
+    assert x.dim() == 2 and x.element_size() == 2 and x.stride(1) == 1
+    tokens, k = x.shape
+    codes = torch.empty((tokens * top_k, k), dtype=torch.int8, device=x.device)
+    scales = torch.empty((tokens * top_k,), dtype=torch.float32, device=x.device)
+    lib = _lib.load()
+    _lib.check(lib.cmx_int8_quant_scatter(_p(x), x.stride(0), _p(src2sorted), _p(codes), k, _p(scales), tokens, k, top_k, _stream()))
+    return codes, scales
+
+
+def int8_gmm_dequant_swiglu(a, token_scale, b, channel_scale, group_sizes, n: int, k: int, trans_b: int = 0,
+                            out: str = "fp32", scale_stride: int = 1, c=None) -> torch.Tensor:
+    """a int8 [rows, k]; b int8 [G, k, n] (trans_b = 0) or [G, n, k] (trans_b = 1); channel_scale fp32 [G*n*scale_stride]."""
+    _need_cuda(a, token_scale, b, channel_scale, group_sizes)
+    assert a.is_contiguous() and b.is_contiguous() and group_sizes.dtype == torch.int32
+    rows, g = a.shape[0], b.shape[0]
+    lib = _lib.load()
+    ws = torch.empty(lib.cmx_int8_gmm_workspace_bytes(g, n, k, trans_b), dtype=torch.uint8, device=a.device)
+    if c is None:
+        c = torch.zeros((rows, n // 2), dtype=_OUT_DTYPE[out], device=a.device)
+    _lib.check(lib.cmx_int8_gmm_dequant_swiglu(_p(a), k, _p(token_scale), _p(b), _p(channel_scale), scale_stride, _p(c),
+                                               c.stride(0), OUT[out], _p(group_sizes), g, rows, n, k, trans_b, _p(ws), _stream()))
+    return c
+
+
 def gmm_workspace(groups: int, device) -> torch.Tensor:
     lib = _lib.load()
     return torch.empty(lib.cmx_mx_gmm_workspace_bytes(groups), dtype=torch.uint8, device=device)

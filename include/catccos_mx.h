@@ -172,6 +172,41 @@ int cmx_mx_gmm_ex(const uint8_t* a, const uint8_t* a_scale, const uint8_t* b, co
                   int fmt, int out_type, int trans_b, void* workspace, cmx_stream_t stream);
 
 /* ------------------------------------------------------------------------------------------
+ * INT8 W8A8 grouped matmul with per-channel and per-token dequantisation and SwiGLU: the arithmetic of the
+ * reference operator DispatchGmmDequantSwiglu.
+ * Replaces AlltoallvGmmDequantKernel + DequantSwigluKernel as composed by AllToAllVGmmDequantSwigluImpl
+ * (examples/dispatch_gmm_dequant_swiglu/dispatch_gmm_dequant_swiglu_device.h:60-222) for the rows one
+ * device holds; golden examples/utils/gen_data_dispatch_gmm_dequant_swiglu.py:263-320:
+ *   c = a_g(int32) @ b_g(int32);  h = fp16(fp32(c) * channel_scale);  y = fp32(h) * token_scale[row];
+ *   out = y[:, :n/2] * sigmoid(y[:, :n/2]) * y[:, n/2:]
+ *
+ *   a              int8 [m_total, k] (expert-sorted rows), pitch lda bytes;  token_scale fp32 [m_total]
+ *   b              int8 [groups, k, n] as the reference stores it (trans_b = 0; rewritten K-contiguous in the
+ *                  workspace on every call) or [groups, n, k] (trans_b = 1, e.g. rewritten once at load time with
+ *                  cmx_bytes_to_k_major)
+ *   channel_scale  fp32 [groups * n], one value every channel_scale_stride floats (2 for the reference's file
+ *                  of 64-bit words whose low half is the fp32 scale, dispatch_gmm_dequant_swiglu_host.h:26,52-61)
+ *   out            [m_total, n/2] of out_type (fp32 as the golden, or fp16 / bf16 as the device writes), pitch
+ *                  ld_out elements;  rows past sum(group_sizes) are left untouched
+ *   workspace      256-byte aligned, cmx_int8_gmm_workspace_bytes bytes
+ * k a multiple of 128, n a multiple of 64.
+ *
+ * cmx_int8_quant_scatter is the per-token dynamic quantiser in front of it (the quant_mode = 1 leg of the routing
+ * routine the golden calls, :159-165; formula :269-274): q = rint(x * 127 / rowmax), scale = rowmax / 127, the row
+ * written to each of its top_k destinations src2sorted[t * top_k + r] (negative = skipped; null = identity with
+ * top_k = 1).  x bf16 [tokens, k].
+ * ---------------------------------------------------------------------------------------- */
+int cmx_int8_quant_scatter(const void* x, uint32_t ld_x, const int32_t* src2sorted, int8_t* codes, uint32_t ld_codes,
+                           float* scales, uint32_t tokens, uint32_t k, uint32_t top_k, cmx_stream_t stream);
+int cmx_bytes_to_k_major(const uint8_t* src, uint32_t ld_src, uint8_t* dst, uint32_t ld_dst, uint32_t k, uint32_t n,
+                         uint32_t batch, cmx_stream_t stream);
+size_t cmx_int8_gmm_workspace_bytes(uint32_t groups, uint32_t n, uint32_t k, int trans_b);
+int cmx_int8_gmm_dequant_swiglu(const int8_t* a, uint32_t lda, const float* token_scale, const int8_t* b,
+                                const float* channel_scale, uint32_t channel_scale_stride, void* out, uint32_t ld_out,
+                                int out_type, const int32_t* group_sizes, uint32_t groups, uint32_t m_total, uint32_t n,
+                                uint32_t k, int trans_b, void* workspace, cmx_stream_t stream);
+
+/* ------------------------------------------------------------------------------------------
  * MoE routing: stable sort of (expert, row) pairs.
  * Replaces moe_init_routing_v2 (examples/aux_ops/moe_init_routing_v2/moe_init_routing_v2.h:56-220,
  * moe_v2_src_to_dst_op_simt.h:79-87); golden moe_init_routing_cpu (gen_data_moe.py:48-57).
