@@ -29,6 +29,7 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBS = 8000.0
 MXFP8_PEAK_TFLOPS = 5000.0
 MXFP4_PEAK_TFLOPS = 10100.0
+INT8_PEAK_TOPS = 5000.0
 SEED = 20240607
 
 
@@ -42,7 +43,7 @@ def main() -> int:
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=30,
                     help="untimed launches first; the launch time keeps falling for about 25 launches after an idle GPU")
-    ap.add_argument("--only", type=str, default="", help="comma list of extras: quant,gemm,ffn,fp4,routing,copycal (default: all but copycal)")
+    ap.add_argument("--only", type=str, default="", help="comma list of extras: quant,gemm,ffn,fp4,int8,routing,copycal (default: all but copycal)")
     ap.add_argument("--no-extras", action="store_true")
     ap.add_argument("--no-cpu", action="store_true")
     args = ap.parse_args()
@@ -125,7 +126,7 @@ def main() -> int:
     flop = 2.0 * rows * H * N
     value = flop / wall / 1e12
     log(f"[gmm1+swiglu+requant cfg3] wall {wall*1e6:.1f} us/step, events {kern*1e6:.1f} us -> {flop/kern/1e12:.0f} TFLOP/s")
-    roofline = {"kernel": "mx_gemm_pipe_kernel<E4M3, swiglu+requant epilogue, 256x256 tile, 4x1 wavefronts, persistent> (grouped, config 3; one launch also runs the 1-workgroup gmm_prepare_kernel)", "bound": "mfma",
+    roofline = {"kernel": "mx_gemm_pipe_kernel<E4M3, swiglu+requant epilogue, 256x256 tile, 2x2 wavefronts, persistent> (grouped, config 3; one launch also runs the 1-workgroup gmm_prepare_kernel)", "bound": "mfma",
                 "achieved": flop / kern / 1e12, "peak": MXFP8_PEAK_TFLOPS, "unit": "TFLOP/s",
                 "frac": flop / kern / 1e12 / MXFP8_PEAK_TFLOPS,
                 # HBM-side bytes per launch from the rocprofv3 --pmc runs summarised under profiles/
@@ -170,7 +171,7 @@ def main() -> int:
 
     # ------------------------------------------------------------------ extras -----------------
     extra = {}
-    want = set(x for x in args.only.split(",") if x) or {"quant", "gemm", "ffn", "fp4", "routing"}
+    want = set(x for x in args.only.split(",") if x) or {"quant", "gemm", "ffn", "fp4", "int8", "routing"}
     if args.no_extras:
         want = set()
 
@@ -221,6 +222,26 @@ def main() -> int:
                                          "bytes_per_launch": bytes_l, "avg_launch_us": tl * 1e6}
         log(f"[mx_to_k_major cfg2 B] {tl*1e6:.1f} us -> {bytes_l/tl/1e9:.0f} GB/s")
         del a2, a2s, b2, b2s, bt, bts
+
+    if "int8" in want:
+        # the reference operator's own arithmetic (INT8 W8A8, per-channel and per-token scales) at config 3's shape
+        g.manual_seed(SEED + 8)
+        a8 = torch.randint(-127, 128, (rows, H), dtype=torch.int8, device=dev, generator=g)
+        ts8 = torch.rand((rows,), device=dev, generator=g) * 1e-2 + 1e-3
+        w8 = torch.randint(-127, 128, (E, N, H), dtype=torch.int8, device=dev, generator=g)      # [E, N, K]: K-contiguous
+        ch8 = torch.rand((E * N,), device=dev, generator=g) * 1e-4
+        o8 = torch.empty((rows, N // 2), dtype=torch.float32, device=dev)
+        t8 = hip_time(lambda: ops.int8_gmm_dequant_swiglu(a8, ts8, w8, ch8, counts, N, H, 1, "fp32", c=o8))
+        extra["int8_gmm_dequant_swiglu_cfg3_shape"] = {
+            "kernel": "mx_gemm_dl_kernel<INT8, dequant+swiglu epilogue, 256x256 tile, 8 wavefronts> (grouped)", "bound": "mfma",
+            "achieved": flop / t8 / 1e12, "peak": INT8_PEAK_TOPS, "unit": "TOP/s", "frac": flop / t8 / 1e12 / INT8_PEAK_TOPS,
+            "avg_launch_us": t8 * 1e6}
+        log(f"[int8 gmm+dequant+swiglu, cfg3 shape] {t8*1e6:.1f} us -> {flop/t8/1e12:.0f} TOP/s")
+        w8t = w8.transpose(1, 2).contiguous()                                                   # [E, K, N] as the reference stores it
+        t8b = hip_time(lambda: ops.int8_gmm_dequant_swiglu(a8, ts8, w8t, ch8, counts, N, H, 0, "fp32", c=o8), steps=max(5, K_STEPS // 4))
+        extra["int8_gmm_dequant_swiglu_cfg3_shape"]["avg_launch_us_k_slow_weights"] = t8b * 1e6
+        log(f"[int8, weights stored [E,K,N] and rewritten per call] {t8b*1e6:.1f} us")
+        del a8, ts8, w8, w8t, ch8, o8
 
     if "fp4" in want:
         E5, T5, K5, N5 = 32, 8192, 7168, 4096

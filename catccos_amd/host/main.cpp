@@ -7,6 +7,8 @@
 //     --data DIR    directory with the operator's input .bin files; outputs are written there too
 //                   (without it inputs are defaults / zeros and nothing is written)
 //     --fmt F       e4m3 | e5m2 | e2m1 | e1m2 for the quantizer, e4m3 | e5m2 for the dense matmul (default e4m3)
+//     --arith A     mx | int8 for DispatchGmmDequantSwiglu (default mx; int8 = the reference operator's own arithmetic
+//                   and file names: a_gm, b_gm, scale_gm, expert_idx -> output)
 //     --transa 0|1  dense matmul: A files hold [K, M] / [K/64, M, 2] when 1 (default 0)
 //     --transb 0|1  dense matmul: B files hold [K, N] / [K/64, N, 2] when 0 (default 1: [N, K])
 //     --repeats R   launches per case (default 1)               --warmup W   untimed launches (default 5)
@@ -24,6 +26,7 @@
 
 #include "launch_map.h"
 #include "ops/ascend950_mxfp8_matmul_reduce_scatter_host.h"
+#include "ops/dispatch_gmm_dequant_swiglu_host.h"
 #include "ops/mx_quant_allgather_host.h"
 
 namespace {
@@ -31,7 +34,7 @@ namespace {
 struct Options {
     std::string op;
     uint32_t m = 0, k = 0, n = 0, experts = 4, topK = 4, repeats = 1, warmup = 5, m0 = M0, transA = 0, transB = 1;
-    std::string data, fmt = "e4m3";
+    std::string data, fmt = "e4m3", arith = "mx";
     bool poison = false;
 };
 
@@ -49,7 +52,7 @@ Options Parse(int argc, char** argv)
 {
     if (argc < 5) {
         throw std::runtime_error("Usage: catccos_mx_run <operator> M K N [--experts E] [--topk T] [--data DIR] [--fmt F] "
-                                 "[--repeats R] [--warmup W] [--poison] [--m0 128|256] [--transa 0|1] [--transb 0|1]");
+                                 "[--repeats R] [--warmup W] [--poison] [--m0 128|256] [--transa 0|1] [--transb 0|1] [--arith mx|int8]");
     }
     Options o;
     o.op = argv[1];
@@ -71,10 +74,12 @@ Options Parse(int argc, char** argv)
         else if (a == "--transb") o.transB = static_cast<uint32_t>(std::strtoul(next("--transb"), nullptr, 10));
         else if (a == "--data") o.data = next("--data");
         else if (a == "--fmt") o.fmt = next("--fmt");
+        else if (a == "--arith") o.arith = next("--arith");
         else if (a == "--poison") o.poison = true;
         else throw std::runtime_error("unknown option " + a);
     }
     if (o.m0 != 128 && o.m0 != 256) throw std::runtime_error("Invalid GMM1 M tile");
+    if (o.arith != "mx" && o.arith != "int8") throw std::runtime_error("unknown arithmetic " + o.arith);
     return o;
 }
 
@@ -106,6 +111,8 @@ int Run(int argc, char** argv)
     }
     const int fmt = FormatOf(o.fmt);
     MxQuantAllGatherOperator::ElementFormat() = fmt;
+    DispatchGmmDequantSwigluOperator::Arithmetic() =
+        o.arith == "int8" ? DispatchGmmDequantSwigluOperator::kInt8 : DispatchGmmDequantSwigluOperator::kMx;
     const bool fp4 = fmt == CMX_FMT_E2M1 || fmt == CMX_FMT_E1M2;
     MxQuantAllGatherOperator::RoundMode() = fp4 ? CMX_ROUND_LUT : CMX_ROUND_RNE;
     Ascend950MxFp8MatmulReduceScatterOperator::ElementFormat() = fp4 ? CMX_FMT_E4M3 : fmt;

@@ -115,6 +115,31 @@ def test_driver_mxfp8_matmul_operand_orientations(host_bin, tmp_path, trans_a, t
 
 
 @pytest.mark.gpu
+def test_driver_int8_dispatch_gmm_dequant_swiglu(host_bin, tmp_path):
+    """The reference operator's own arithmetic and file names (examples/dispatch_gmm_dequant_swiglu/
+    dispatch_gmm_dequant_swiglu_host.h:31-73): a_gm bf16 [m, k], b_gm int8 [E, k, n], scale_gm 64-bit words,
+    expert_idx int32 [m, topK] -> output bf16 [m * topK, n / 2], rows sorted by expert."""
+    from oracle import int8_oracle as Q
+    m, k, n, experts, top_k = 48, 512, 256, 4, 4
+    rng = np.random.default_rng(31)
+    x = W.normal_bf16((m, k), 6)
+    idx = rng.integers(0, experts, size=(m, top_k)).astype(np.int32)
+    b = rng.integers(-16, 16, size=(experts, k, n), dtype=np.int8)
+    ch = Q.truncate_scale(rng.standard_normal(experts * n).astype(np.float32) / 127)
+    for stem, arr in (("a_gm", x), ("b_gm", b), ("scale_gm", Q.channel_scale_words(ch)), ("expert_idx", idx)):
+        _write(tmp_path / f"{stem}_0.bin", arr)
+    r = _run(host_bin, "DispatchGmmDequantSwiglu", m, k, n, "--experts", experts, "--topk", top_k, "--data", tmp_path,
+             "--arith", "int8", "--poison")
+    assert r.returncode == 0, r.stdout + r.stderr
+    sorted2src = np.argsort(idx.reshape(-1), kind="stable")
+    counts = np.bincount(idx.reshape(-1), minlength=experts)
+    aq, ts = Q.dispatch_quant(O.bf16_bits_to_f32(x), sorted2src, top_k)
+    gold = Q.gmm_dequant_swiglu(aq, ts, b, ch, counts)
+    got = O.bf16_bits_to_f32(np.fromfile(tmp_path / "output_0.bin", dtype=np.uint16).reshape(m * top_k, n // 2))
+    assert np.allclose(got, gold, rtol=1e-2, atol=1e-3)
+
+
+@pytest.mark.gpu
 def test_driver_ffn(host_bin, tmp_path):
     tokens, k, n, experts, top_k = 64, 512, 1024, 8, 4
     rng = np.random.default_rng(3)
