@@ -20,6 +20,7 @@
 // that prefix, so no host synchronisation is needed and empty groups cost nothing.  Workgroup ids
 // are remapped so that each XCD (ids congruent mod 8) walks a contiguous run of tiles that share
 // weight panels in its own L2.
+#include <atomic>
 #include <type_traits>
 
 #include "mx_common.h"
@@ -835,45 +836,111 @@ __global__ __launch_bounds__(64 * WW * WM) void mx_gemm_dl_kernel(const GemmPara
 
 #include "mx_gemm_pipe.h"
 
-// Row offsets and m-tile prefix of the groups (one workgroup of 256 threads): each thread sums a contiguous
-// run of groups, the 256 partial sums are scanned in LDS, and each thread writes its run.
+// Row offsets and m-tile prefix of the groups (one workgroup of 256 threads): each thread owns a contiguous run of
+// groups; the 256 partial sums are scanned in LDS, first for the rows, then for the m-tiles.
+// Group sizes live on the device, so the host cannot check them: negative sizes count as zero and rows past
+// m_total (the rows the caller's buffers hold) are cut off here, so that no tile ever points outside them.
 __global__ __launch_bounds__(256) void gmm_prepare_kernel(const int32_t* __restrict__ sizes, uint32_t groups, uint32_t tile_m,
-                                                           int32_t* __restrict__ row_off, int32_t* __restrict__ tile_pref,
-                                                           int32_t* __restrict__ tile_ctr) {
-    __shared__ int32_t part_r[256], part_t[256];
+                                                           uint32_t m_total, int32_t* __restrict__ row_off,
+                                                           int32_t* __restrict__ tile_pref, int32_t* __restrict__ tile_ctr) {
+    __shared__ unsigned long long part_r[256];
+    __shared__ int32_t part_t[256];
     if (threadIdx.x < kXcds) tile_ctr[threadIdx.x] = 0;
     const uint32_t per = (groups + 255) / 256;
-    const uint32_t lo = threadIdx.x * per, hi = lo + per < groups ? lo + per : groups;
-    int32_t r = 0, t = 0;
-    for (uint32_t i = lo; i < hi; ++i) {
-        const int32_t c = sizes[i] > 0 ? sizes[i] : 0;
-        r += c;
-        t += (c + (int32_t)tile_m - 1) / (int32_t)tile_m;
-    }
+    const uint32_t lo = threadIdx.x * per < groups ? threadIdx.x * per : groups;
+    const uint32_t hi = lo + per < groups ? lo + per : groups;
+    auto size_of = [&](uint32_t i) -> unsigned long long {
+        const int32_t c = sizes[i];
+        return c > 0 ? (unsigned long long)c : 0ull;
+    };
+    auto scan256 = [&](auto* part) {
+        for (uint32_t d = 1; d < 256; d <<= 1) {
+            const auto v = threadIdx.x >= d ? part[threadIdx.x - d] : 0;
+            __syncthreads();
+            part[threadIdx.x] += v;
+            __syncthreads();
+        }
+    };
+    unsigned long long r = 0;
+    for (uint32_t i = lo; i < hi; ++i) r += size_of(i);
     part_r[threadIdx.x] = r;
+    __syncthreads();
+    scan256(part_r);
+    const unsigned long long r_base = threadIdx.x ? part_r[threadIdx.x - 1] : 0ull;
+    // rows of group i that fit below m_total, given the rows before it
+    auto clipped = [&](unsigned long long before, unsigned long long c) -> uint32_t {
+        const unsigned long long b = before < m_total ? before : m_total;
+        const unsigned long long e = before + c < m_total ? before + c : m_total;
+        return (uint32_t)(e - b);
+    };
+    r = r_base;
+    int32_t t = 0;
+    for (uint32_t i = lo; i < hi; ++i) {
+        const unsigned long long c = size_of(i);
+        t += (int32_t)((clipped(r, c) + tile_m - 1) / tile_m);
+        r += c;
+    }
     part_t[threadIdx.x] = t;
     __syncthreads();
-    for (uint32_t d = 1; d < 256; d <<= 1) {
-        const int32_t vr = threadIdx.x >= d ? part_r[threadIdx.x - d] : 0;
-        const int32_t vt = threadIdx.x >= d ? part_t[threadIdx.x - d] : 0;
-        __syncthreads();
-        part_r[threadIdx.x] += vr;
-        part_t[threadIdx.x] += vt;
-        __syncthreads();
-    }
-    r = threadIdx.x ? part_r[threadIdx.x - 1] : 0;
+    scan256(part_t);
+    r = r_base;
     t = threadIdx.x ? part_t[threadIdx.x - 1] : 0;
     for (uint32_t i = lo; i < hi; ++i) {
-        const int32_t c = sizes[i] > 0 ? sizes[i] : 0;
-        row_off[i] = r;
+        const unsigned long long c = size_of(i);
+        row_off[i] = (int32_t)(r < m_total ? r : m_total);
         tile_pref[i] = t;
+        t += (int32_t)((clipped(r, c) + tile_m - 1) / tile_m);
         r += c;
-        t += (c + (int32_t)tile_m - 1) / (int32_t)tile_m;
     }
     if (threadIdx.x == 255) {
-        row_off[groups] = part_r[255];
+        const unsigned long long all = part_r[255];
+        row_off[groups] = (int32_t)(all < m_total ? all : m_total);
         tile_pref[groups] = part_t[255];
     }
+}
+
+// Launch state that belongs to a device, not to the process: the dynamic-LDS limit of a kernel has to be raised on
+// every device that runs it, and the CU count differs between devices.  One slot per device ordinal; the flags are
+// atomics so that concurrent first calls from several host threads are merely redundant.
+constexpr int kMaxDevices = 64;
+
+struct PerDeviceFlag {
+    std::atomic<bool> done[kMaxDevices];
+};
+
+int current_device_slot(int* dev_out) {
+    int dev = 0;
+    CMX_HIP(hipGetDevice(&dev));
+    CMX_REQUIRE(dev >= 0 && dev < kMaxDevices, "device ordinal out of range");
+    *dev_out = dev;
+    return CMX_OK;
+}
+
+template <typename K>
+int allow_dynamic_lds(K kfn, size_t bytes, PerDeviceFlag& flag) {
+    int dev = 0;
+    int rc = current_device_slot(&dev);
+    if (rc != CMX_OK) return rc;
+    if (!flag.done[dev].load(std::memory_order_acquire)) {
+        CMX_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kfn), hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes));
+        flag.done[dev].store(true, std::memory_order_release);
+    }
+    return CMX_OK;
+}
+
+int cu_count(int* out) {
+    static std::atomic<int> cus[kMaxDevices];
+    int dev = 0;
+    int rc = current_device_slot(&dev);
+    if (rc != CMX_OK) return rc;
+    int n = cus[dev].load(std::memory_order_acquire);
+    if (n == 0) {
+        CMX_HIP(hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev));
+        n = n > 0 ? n : 256;
+        cus[dev].store(n, std::memory_order_release);
+    }
+    *out = n;
+    return CMX_OK;
 }
 
 template <int FMT, int TW, int TM, int WW, int WM, int EPI, bool FAST>
@@ -881,12 +948,8 @@ int launch_gemm_impl(const GemmParams& p, uint32_t max_m_tiles, hipStream_t s) {
     constexpr int kScaleDw = FMT == CMX_FMT_E2M1 ? 2 : 1;
     constexpr size_t smem = 2 * ((TW + TM) * kSlabBytes + (TW + TM) * 4 * kScaleDw);
     auto kfn = mx_gemm_kernel<FMT, TW, TM, WW, WM, EPI, FAST>;
-    static bool attr_set = false;
-    if (!attr_set) {
-        CMX_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kfn), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                    (int)smem));
-        attr_set = true;
-    }
+    static PerDeviceFlag lds_allowed;
+    if (int rc = allow_dynamic_lds(kfn, smem, lds_allowed); rc != CMX_OK) return rc;
     const uint64_t tiles = (uint64_t)max_m_tiles * p.w_tiles;
     CMX_REQUIRE(tiles > 0 && tiles < (1ull << 31), "tile count out of range");
     hipLaunchKernelGGL(kfn, dim3((uint32_t)tiles), dim3(64 * WW * WM), smem, s, p);
@@ -899,12 +962,8 @@ int launch_gemm_dl(const GemmParams& p, uint32_t max_m_tiles, hipStream_t s) {
     constexpr int kScaleDw = FMT == CMX_FMT_E2M1 ? 2 : 1;
     constexpr size_t smem = 2 * (TW + TM) * kSlabBytes + 2 * (TW + TM) * kScaleDw * 4;
     auto kfn = mx_gemm_dl_kernel<FMT, TW, TM, WW, WM, EPI>;
-    static bool attr_set = false;
-    if (!attr_set) {
-        CMX_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kfn), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                    (int)smem));
-        attr_set = true;
-    }
+    static PerDeviceFlag lds_allowed;
+    if (int rc = allow_dynamic_lds(kfn, smem, lds_allowed); rc != CMX_OK) return rc;
     const uint64_t tiles = (uint64_t)max_m_tiles * p.w_tiles;
     CMX_REQUIRE(tiles > 0 && tiles < (1ull << 31), "tile count out of range");
     hipLaunchKernelGGL(kfn, dim3((uint32_t)tiles), dim3(64 * WW * WM), smem, s, p);
@@ -917,24 +976,15 @@ int launch_gemm_pipe(const GemmParams& p, uint32_t max_m_tiles, hipStream_t s) {
     // tile ring, scale ring (two-slot kernels: two blocks of 16 bytes per row), next-tile mailbox
     constexpr size_t smem = NSLOT * (256 + TM) * kSlabBytes + (NSLOT == 2 ? 2 * (256 + TM) * 16 : NSLOT * (256 + TM) * 4) + 16;
     auto kfn = mx_gemm_pipe_kernel<FMT, EPI, TM, WW, WM, NSLOT>;
-    static bool attr_set = false;
-    if (!attr_set) {
-        CMX_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kfn), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                    (int)smem));
-        attr_set = true;
-    }
+    static PerDeviceFlag lds_allowed;
+    if (int rc = allow_dynamic_lds(kfn, smem, lds_allowed); rc != CMX_OK) return rc;
     const uint64_t tiles = (uint64_t)max_m_tiles * p.w_tiles;
     CMX_REQUIRE(tiles > 0 && tiles < (1ull << 31), "tile count out of range");
     uint32_t grid = (uint32_t)tiles;
     if (pipe_is_persistent(NSLOT, EPI)) {
         // persistent: one workgroup per CU (the LDS footprint admits no second one), a multiple of the XCD count
-        static int cus = 0;
-        if (cus == 0) {
-            int dev = 0, n = 0;
-            CMX_HIP(hipGetDevice(&dev));
-            CMX_HIP(hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev));
-            cus = n > 0 ? n : 256;
-        }
+        int cus = 0;
+        if (int rc = cu_count(&cus); rc != CMX_OK) return rc;
         grid = (uint32_t)(cus / kXcds * kXcds);
         if (grid < (uint32_t)kXcds) grid = kXcds;
     }
@@ -1095,6 +1145,7 @@ int gmm_common(GemmParams& p, const int32_t* group_sizes, uint32_t groups, uint3
                bool swiglu, hipStream_t s) {
     CMX_REQUIRE(group_sizes && workspace, "null pointer");
     CMX_REQUIRE(groups > 0 && groups <= 65536, "bad group count");
+    CMX_REQUIRE(m_total < (1u << 31), "too many rows");
     CMX_REQUIRE((uint64_t)p.n * p.ldw < (1ull << 32) && (uint64_t)p.lda * 256 < (1ull << 32),
                 "operand tile exceeds 32-bit offsets");
     CMX_REQUIRE((reinterpret_cast<uintptr_t>(workspace) & 3u) == 0, "workspace must be 4-byte aligned");
@@ -1103,8 +1154,8 @@ int gmm_common(GemmParams& p, const int32_t* group_sizes, uint32_t groups, uint3
     int32_t* row_off = static_cast<int32_t*>(workspace);
     int32_t* tile_pref = row_off + (groups + 1);
     int32_t* tile_ctr = tile_pref + (groups + 1);
-    hipLaunchKernelGGL(gmm_prepare_kernel, dim3(1), dim3(256), 0, s, group_sizes, groups, (uint32_t)t.tm, row_off, tile_pref,
-                       tile_ctr);
+    hipLaunchKernelGGL(gmm_prepare_kernel, dim3(1), dim3(256), 0, s, group_sizes, groups, (uint32_t)t.tm, m_total, row_off,
+                       tile_pref, tile_ctr);
     CMX_LAUNCH_CHECK();
     p.row_off = row_off;
     p.tile_pref = tile_pref;
@@ -1155,7 +1206,7 @@ extern "C" int cmx_int8_gmm_dequant_swiglu(const int8_t* a, uint32_t lda, const 
     using namespace cmx;
     if (m_total == 0 || n == 0) return CMX_OK;
     CMX_REQUIRE(a && token_scale && b && channel_scale && out && group_sizes && workspace, "null pointer");
-    CMX_REQUIRE(groups > 0 && groups <= 65536, "bad group count");
+    CMX_REQUIRE(groups > 0 && groups <= 65536 && m_total < (1u << 31), "bad group count or too many rows");
     CMX_REQUIRE(k > 0 && k % kSlabBytes == 0 && k < (1u << 17), "k must be a multiple of 128 below 131072 (INT32 accumulation)");
     CMX_REQUIRE(n % 64 == 0, "n must be a multiple of 64 (32-wide gate and up fragments)");
     CMX_REQUIRE(lda >= k && lda % 16 == 0 && aligned16(a) && aligned16(b), "operand rows must be 16-byte aligned");
@@ -1186,8 +1237,8 @@ extern "C" int cmx_int8_gmm_dequant_swiglu(const int8_t* a, uint32_t lda, const 
     int32_t* tile_pref = row_off + (groups + 1);
     int32_t* tile_ctr = tile_pref + (groups + 1);
     constexpr int kTile = 256;
-    hipLaunchKernelGGL(gmm_prepare_kernel, dim3(1), dim3(256), 0, s, group_sizes, groups, (uint32_t)kTile, row_off, tile_pref,
-                       tile_ctr);
+    hipLaunchKernelGGL(gmm_prepare_kernel, dim3(1), dim3(256), 0, s, group_sizes, groups, (uint32_t)kTile, m_total, row_off,
+                       tile_pref, tile_ctr);
     CMX_LAUNCH_CHECK();
     p.row_off = row_off;
     p.tile_pref = tile_pref;

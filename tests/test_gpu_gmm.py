@@ -71,6 +71,25 @@ def test_gmm_many_ragged_groups_every_row(tile):
     assert np.array_equal(host(scales), ws2) and np.array_equal(host(codes), wq2)
 
 
+@pytest.mark.parametrize("tile", [None, (256, 128, 5), (128, 128, 4)])
+def test_group_sizes_that_overrun_the_buffers_are_cut_off(tile):
+    """The sizes are device data the host cannot check: rows past m_total are dropped group by group and negative
+    sizes count as zero, so the kernels never leave the caller's buffers."""
+    from catccos_amd import ops, _lib
+    if tile:
+        _lib.load().cmx_debug_force_tile(*tile)
+    rng = np.random.default_rng(41)
+    n, k, m = 192, 512, 400
+    aq, asc = O.mx_quant(O.bf16_round(rng.standard_normal((m, k)).astype(np.float32)))
+    wq, ws = _weights(rng, 4, n, k, std=1.0)
+    claimed = np.array([300, -5, 300, 1 << 30], dtype=np.int32)          # only 300 + 100 rows exist
+    c = torch.full((m, n), 7.0, dtype=torch.bfloat16, device="cuda")
+    ops.mx_gmm(dev(aq), dev(asc), dev(wq), dev(ws), dev(claimed), k, c=c)
+    gold = O.mx_gmm_f32(aq, asc, wq, ws, [300, 0, 100, 0])
+    bad, worst = close_bf16(host(c), gold)
+    assert bad == 0, (bad, worst)
+
+
 def test_gmm_fp4_ragged_groups():
     from catccos_amd import ops
     rng = np.random.default_rng(3)
