@@ -42,3 +42,24 @@ def test_host_only_entry_points_work_without_a_gpu():
     # a bad argument is reported through the error string, not a crash
     rc = lib.cmx_mx_quant(None, 0, None, 0, None, 0, 1, 33, 0, 0, None)
     assert rc != 0 and lib.cmx_last_error()
+
+
+def test_header_is_plain_c(tmp_path):
+    """The boundary is a C ABI: the header must compile as C99 (and as C++) on its own."""
+    import subprocess
+    for compiler, std, lang in (("gcc", "-std=c99", "c"), ("g++", "-std=c++17", "c++")):
+        r = subprocess.run([compiler, std, "-Wall", "-Wextra", "-Werror", "-fsyntax-only", "-x", lang, HEADER],
+                           capture_output=True, text=True)
+        assert r.returncode == 0, r.stderr
+
+
+def test_workspace_sizes_are_host_arithmetic():
+    from catccos_amd import _lib
+    lib = _lib.load()
+    assert lib.cmx_mx_gemm_ex_workspace_bytes(100, 200, 512, 0, 1) == 0                    # both operands K-contiguous
+    need = lib.cmx_mx_gemm_ex_workspace_bytes(100, 200, 512, 1, 0)
+    assert need >= (100 + 200) * (512 + 16) and need % 256 == 0
+    meta = lib.cmx_mx_gmm_workspace_bytes(16)
+    assert lib.cmx_mx_gmm_ex_workspace_bytes(16, 256, 512, 1) >= meta
+    assert lib.cmx_mx_gmm_ex_workspace_bytes(16, 256, 512, 0) >= meta + 16 * 256 * (512 + 16)
+    assert lib.cmx_int8_gmm_workspace_bytes(4, 256, 512, 0) >= lib.cmx_int8_gmm_workspace_bytes(4, 256, 512, 1) + 4 * 256 * 512
