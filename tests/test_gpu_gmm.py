@@ -90,6 +90,44 @@ def test_group_sizes_that_overrun_the_buffers_are_cut_off(tile):
     assert bad == 0, (bad, worst)
 
 
+@pytest.mark.parametrize("fmt", ["E4M3", "E5M2"])
+def test_groups_about_one_tile_long(fmt):
+    """Average group size between 128 and 512 rows with the default dispatch (256-row tiles, 4 x 1 wavefronts):
+    remainders of 1, 64, 65, 128 and 129 rows past whole tiles, groups below and above one tile."""
+    from catccos_amd import ops
+    rng = np.random.default_rng(53)
+    counts = [257, 256, 100, 320, 384, 385, 0, 250, 513, 129, 64, 300]
+    assert 128 < sum(counts) / len(counts) < 512
+    n, k = 320, 512
+    m = sum(counts)
+    aq, asc = O.mx_quant(O.bf16_round(rng.standard_normal((m + 5, k)).astype(np.float32)), fmt)
+    qs = [O.mx_quant(O.bf16_round(rng.standard_normal((n, k)).astype(np.float32)), fmt, "rne") for _ in counts]
+    wq, ws = np.stack([q for q, _ in qs]), np.stack([s_ for _, s_ in qs])
+    c = torch.full((m + 5, n), 7.0, dtype=torch.bfloat16, device="cuda")
+    ops.mx_gmm(dev(aq), dev(asc), dev(wq), dev(ws), dev(np.array(counts, dtype=np.int32)), k, fmt, c=c)
+    got = host(c)
+    bad, worst = close_bf16(got[:m], O.mx_gmm_f32(aq[:m], asc[:m], wq, ws, counts, fmt, fmt))
+    assert bad == 0, (bad, worst)
+    assert np.all(O.bf16_bits_to_f32(got[m:]) == 7.0)
+
+
+def test_swiglu_requant_with_groups_about_one_tile_long():
+    from catccos_amd import ops
+    rng = np.random.default_rng(54)
+    counts = [257, 256, 100, 320, 384, 385, 0, 250, 513, 129, 64, 300]
+    n, k = 512, 512
+    m = sum(counts)
+    aq, asc = O.mx_quant(O.bf16_round(rng.standard_normal((m, k)).astype(np.float32)))
+    wq, ws = _weights(rng, len(counts), n, k, std=0.06)
+    codes, scales, act = ops.mx_gmm_swiglu_quant(dev(aq), dev(asc), dev(wq), dev(ws), dev(np.array(counts, dtype=np.int32)), k,
+                                                 want_bf16=True)
+    _, act_g, _, _ = O.gmm1_swiglu_quant(aq, asc, wq, ws, counts)
+    bad, worst = close_bf16(host(act), O.bf16_bits_to_f32(act_g), rtol=2e-2)
+    assert bad == 0, (bad, worst)
+    wq2, ws2 = O.mx_quant_bf16(host(act), "E4M3", "rne")
+    assert np.array_equal(host(scales), ws2) and np.array_equal(host(codes), wq2)
+
+
 def test_gmm_fp4_ragged_groups():
     from catccos_amd import ops
     rng = np.random.default_rng(3)
