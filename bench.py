@@ -2,7 +2,7 @@
 """Benchmark of the MI355X MX compute core (one GPU).
 
 Headline step = one pass of the MoE grouped matmul with fused dequant + SwiGLU + MX requant
-(BASELINE.json config 3: E=16 local experts, 4096 tokens x top-8 Zipf-routed = 32768 ragged rows,
+(the headline configuration, "config 3": E=16 local experts, 4096 tokens x top-8 Zipf-routed = 32768 ragged rows,
 H=7168, W_gate/up [16, 4096, 7168] MXFP8) through the C ABI, inputs resident in HBM.
 `value` = 2*rows*K*N flop / step time in TFLOP/s.  The same JSON line carries
 

@@ -82,3 +82,36 @@ def test_ffn_rejects_bad_shapes():
     assert lib.catccos_ascend950_dispatch_ffn_combine(*args(4, 256, 256, 4, 2, 1)) == -1     # N % 512
     assert lib.catccos_ascend950_dispatch_ffn_combine(*args(4, 256, 512, 4, 5, 1)) == -1     # topK > experts
     assert lib.catccos_ascend950_dispatch_ffn_combine(*args(4, 256, 512, 4, 2, 2)) == -1     # rankSize
+
+
+def test_ffn_chain_replays_from_a_hip_graph():
+    """The chain makes no allocation, no memset and no host synchronisation, so it can be captured into a HIP
+    graph once and replayed: three replays, each after the program changed the tokens in place and did eager work
+    of its own, every one compared bit for bit with an eager run on the same inputs."""
+    from catccos_amd import ops
+    tokens, k, n, experts, top_k = 96, 512, 512, 8, 4
+    x, idx, p, w1q, w1s, w2q, w2s = _make(tokens, k, n, experts, top_k, seed=77)
+    xd, idxd, pd = bf16_dev(x), dev(idx), dev(p)
+    w1d, w1sd, w2d, w2sd = dev(w1q), dev(w1s), dev(w2q), dev(w2s)
+    ws = torch.empty(ops.ffn_workspace_bytes(tokens, k, n, experts, top_k), dtype=torch.uint8, device="cuda")
+    ws_eager = torch.empty_like(ws)
+    out = torch.zeros((tokens, k), dtype=torch.bfloat16, device="cuda")
+    run = lambda o, w: ops.dispatch_ffn_combine(xd, idxd, pd, w1d, w1sd, w2d, w2sd, workspace=w, out=o)
+    run(out, ws)                                   # first launches set kernel attributes: outside the capture
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            run(out, ws)
+    torch.cuda.current_stream().wait_stream(side)
+    for rep in range(3):
+        xd.copy_(bf16_dev(W.normal_bf16((tokens, k), 100 + rep)))       # new tokens in the captured buffer
+        expect = torch.zeros_like(out)
+        run(expect, ws_eager)                      # eager work between the replays
+        torch.cuda.synchronize()
+        out.fill_(7.0)
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out.view(torch.int16), expect.view(torch.int16)), rep

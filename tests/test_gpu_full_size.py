@@ -1,4 +1,4 @@
-"""The BASELINE configurations at their full sizes: sampled rows against the oracle plus properties that
+"""The benchmark configurations 2-5 at their full sizes: sampled rows against the oracle plus properties that
 do not depend on the size (exact scale linearity, row-permutation equivariance, gate-weight linearity).
 Inputs are generated and quantised on the GPU; only the sampled rows travel to the host for the oracle."""
 import numpy as np
