@@ -46,6 +46,7 @@ SIGNATURES = {
     "cmx_mx_gmm_swiglu_quant": (i32, [u8p, u32, u8p, u32, u8p, u8p, u8p, u32, u8p, u32, vp, i32p, u32, u32, u32, u32,
                                       vp, vp]),
     "cmx_mx_to_k_major": (i32, [u8p, u32, u8p, u8p, u32, u8p, u32, u32, u32, u32, vp]),
+    "cmx_mxfp4_to_k_major": (i32, [u8p, u32, u8p, u8p, u32, u8p, u32, u32, u32, u32, vp]),
     "cmx_mx_gemm_ex_workspace_bytes": (sz, [u32, u32, u32, i32, i32]),
     "cmx_mx_gemm_ex": (i32, [u8p, u8p, u8p, u8p, vp, u32, u32, u32, u32, i32, i32, i32, i32, vp, vp]),
     "cmx_mx_gmm_ex_workspace_bytes": (sz, [u32, u32, u32, i32]),

@@ -109,6 +109,118 @@ __global__ __launch_bounds__(256) void mx_to_k_major_kernel(const uint8_t* __res
     }
 }
 
+// FP4: two codes share a byte along the contiguous axis, so the same change of orientation is a transpose of 4-bit
+// units: source [K, N/2] bytes (N pairs per byte, even column in the low nibble) -> destination [N, K/2] bytes (K pairs
+// per byte).  A thread transposes an 8 x 8 block of nibbles held in eight dwords with the three-level masked-swap
+// network (4-, 8- and 16-bit fields); a workgroup moves 128 (K) x 128 (N) codes.
+__device__ __forceinline__ void transpose8x8_nibbles(uint32_t (&w)[8]) {
+#pragma unroll
+    for (int i = 0; i < 8; i += 2) {
+        const uint32_t t = ((w[i] >> 4) ^ w[i + 1]) & 0x0F0F0F0Fu;
+        w[i + 1] ^= t;
+        w[i] ^= t << 4;
+    }
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        if (i & 2) continue;
+        const uint32_t t = ((w[i] >> 8) ^ w[i + 2]) & 0x00FF00FFu;
+        w[i + 2] ^= t;
+        w[i] ^= t << 8;
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const uint32_t t = ((w[i] >> 16) ^ w[i + 4]) & 0x0000FFFFu;
+        w[i + 4] ^= t;
+        w[i] ^= t << 16;
+    }
+}
+
+// grid: (ceil(n / 128), ceil(k / 128), batch); ld_src / ld_dst in bytes
+__global__ __launch_bounds__(256) void mxfp4_to_k_major_kernel(const uint8_t* __restrict__ src, uint32_t ld_src,
+                                                               const uint8_t* __restrict__ src_scale,
+                                                               uint8_t* __restrict__ dst, uint32_t ld_dst,
+                                                               uint8_t* __restrict__ dst_scale, uint32_t ld_dst_scale,
+                                                               uint32_t k, uint32_t n, uint64_t src_batch,
+                                                               uint64_t dst_batch, uint64_t src_scale_batch,
+                                                               uint64_t dst_scale_batch, int vec_in) {
+    constexpr int kPitch = 16 + 1;                       // dwords per staged destination row (128 K codes = 64 bytes)
+    __shared__ uint32_t tile[kLt * kPitch];              // [n][k / 8]
+    const uint32_t t = threadIdx.x;
+    const uint32_t n0 = blockIdx.x * kLt, k0 = blockIdx.y * kLt;
+    src += blockIdx.z * src_batch;
+    dst += blockIdx.z * dst_batch;
+    src_scale += blockIdx.z * src_scale_batch;
+    dst_scale += blockIdx.z * dst_scale_batch;
+    const uint32_t src_row_bytes = (n + 1) / 2;
+
+    // load: thread -> 8 K rows (kb) x 8 N codes (nb): one dword of each row
+    const uint32_t nb = t & 15u, kb = t >> 4;
+    const uint32_t byte0 = n0 / 2 + 4 * nb;
+    uint32_t w[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+        const uint32_t kr = k0 + 8 * kb + j;
+        w[j] = 0;
+        if (kr < k) {
+            const uint8_t* p = src + (size_t)kr * ld_src + byte0;
+            if (vec_in && byte0 + 4 <= src_row_bytes) {
+                w[j] = *reinterpret_cast<const uint32_t*>(p);
+            } else {
+#pragma unroll
+                for (int b = 0; b < 4; ++b)
+                    if (byte0 + b < src_row_bytes) w[j] |= (uint32_t)p[b] << (8 * b);
+            }
+        }
+    }
+    transpose8x8_nibbles(w);                             // w[i] = codes k0 + 8 kb .. + 7 of column n0 + 8 nb + i
+#pragma unroll
+    for (int i = 0; i < 8; ++i) tile[(8 * nb + i) * kPitch + kb] = w[i];
+    __syncthreads();
+
+    // store: thread -> 16 bytes (32 K codes) of row n0 + t / 4 + 64 i; k is a multiple of 64, so a piece is whole or absent
+    const uint32_t part = t & 3u;
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+        const uint32_t nr = (t >> 2) + 64 * i;
+        const uint32_t kc = k0 + 32 * part;
+        if (n0 + nr < n && kc < k) {
+            const uint32_t* q = tile + nr * kPitch + 4 * part;
+            *reinterpret_cast<uint4*>(dst + (size_t)(n0 + nr) * ld_dst + kc / 2) = make_uint4(q[0], q[1], q[2], q[3]);
+        }
+    }
+
+    // scales: as for the 8-bit formats
+    if (t < (uint32_t)kLt && n0 + t < n) {
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            const uint32_t pair = k0 / 64 + h;
+            if (pair * 64 < k) {
+                const uint8_t* sp = src_scale + ((size_t)pair * n + n0 + t) * 2;
+                uint8_t* dp = dst_scale + (size_t)(n0 + t) * ld_dst_scale + 2 * pair;
+                dp[0] = sp[0];
+                dp[1] = sp[1];
+            }
+        }
+    }
+}
+
+int fp4_to_k_major(const uint8_t* src, uint32_t ld_src, const uint8_t* src_scale, uint8_t* dst, uint32_t ld_dst,
+                   uint8_t* dst_scale, uint32_t ld_dst_scale, uint32_t k, uint32_t n, uint32_t batch, hipStream_t s) {
+    CMX_REQUIRE(src && src_scale && dst && dst_scale, "null pointer");
+    CMX_REQUIRE(k > 0 && k % 64 == 0, "k must be a positive multiple of 64 (scale bytes come in pairs of K blocks)");
+    CMX_REQUIRE(ld_src >= (n + 1) / 2 && ld_dst >= k / 2 && ld_dst_scale >= k / 32, "row pitch smaller than a row");
+    CMX_REQUIRE(ld_dst % 16 == 0 && aligned16(dst), "destination rows must be 16-byte aligned");
+    if (n == 0 || batch == 0) return CMX_OK;
+    CMX_REQUIRE(batch <= 65535u && ceil_div(k, kLt) <= 65535u, "too many tiles for one launch");
+    const int vec_in = ld_src % 4 == 0 && (reinterpret_cast<uintptr_t>(src) & 3u) == 0;
+    dim3 grid(ceil_div(n, kLt), ceil_div(k, kLt), batch);
+    hipLaunchKernelGGL(mxfp4_to_k_major_kernel, grid, dim3(256), 0, s, src, ld_src, src_scale, dst, ld_dst, dst_scale,
+                       ld_dst_scale, k, n, (uint64_t)k * ld_src, (uint64_t)n * ld_dst, (uint64_t)(k / 32) * n,
+                       (uint64_t)n * ld_dst_scale, vec_in);
+    CMX_LAUNCH_CHECK();
+    return CMX_OK;
+}
+
 int to_k_major(const uint8_t* src, uint32_t ld_src, const uint8_t* src_scale, uint8_t* dst, uint32_t ld_dst,
                uint8_t* dst_scale, uint32_t ld_dst_scale, uint32_t k, uint32_t n, uint32_t batch, hipStream_t s) {
     CMX_REQUIRE(src && dst && (src_scale == nullptr) == (dst_scale == nullptr), "null pointer");
@@ -131,7 +243,8 @@ struct ExLayout {
     size_t a_codes, a_scales, b_codes, b_scales, total;
 };
 
-ExLayout ex_layout(uint64_t a_rows, uint64_t b_rows, uint32_t k, int trans_a, int b_k_major) {
+ExLayout ex_layout(uint64_t a_rows, uint64_t b_rows, uint32_t k, int trans_a, int b_k_major, int fmt = CMX_FMT_E4M3) {
+    const uint32_t kbytes = fmt == CMX_FMT_E2M1 ? k / 2 : k;
     ExLayout L{};
     size_t off = 0;
     auto take = [&](size_t bytes) {
@@ -140,11 +253,11 @@ ExLayout ex_layout(uint64_t a_rows, uint64_t b_rows, uint32_t k, int trans_a, in
         return at;
     };
     if (trans_a) {
-        L.a_codes = take(a_rows * k);
+        L.a_codes = take(a_rows * kbytes);
         L.a_scales = take(a_rows * (k / 32));
     }
     if (!b_k_major) {
-        L.b_codes = take(b_rows * k);
+        L.b_codes = take(b_rows * kbytes);
         L.b_scales = take(b_rows * (k / 32));
     }
     L.total = off;
@@ -152,6 +265,15 @@ ExLayout ex_layout(uint64_t a_rows, uint64_t b_rows, uint32_t k, int trans_a, in
 }
 
 bool fmt_is_8bit(int fmt) { return fmt == CMX_FMT_E4M3 || fmt == CMX_FMT_E5M2; }
+bool fmt_has_layouts(int fmt) { return fmt_is_8bit(fmt) || fmt == CMX_FMT_E2M1; }
+
+// operand [k, rows] in the format's K-slow storage -> K-contiguous, packed pitches
+int normalise(const uint8_t* src, const uint8_t* src_scale, uint8_t* dst, uint8_t* dst_scale, uint32_t k, uint32_t rows,
+              uint32_t batch, int fmt, hipStream_t s) {
+    if (fmt == CMX_FMT_E2M1)
+        return fp4_to_k_major(src, (rows + 1) / 2, src_scale, dst, k / 2, dst_scale, k / 32, k, rows, batch, s);
+    return to_k_major(src, rows, src_scale, dst, k, dst_scale, k / 32, k, rows, batch, s);
+}
 
 }  // namespace
 }  // namespace cmx
@@ -165,6 +287,13 @@ extern "C" int cmx_mx_to_k_major(const uint8_t* src, uint32_t ld_src, const uint
     }
     return cmx::to_k_major(src, ld_src, src_scale, dst, ld_dst, dst_scale, ld_dst_scale, k, n, batch,
                            static_cast<hipStream_t>(stream));
+}
+
+extern "C" int cmx_mxfp4_to_k_major(const uint8_t* src, uint32_t ld_src, const uint8_t* src_scale, uint8_t* dst,
+                                    uint32_t ld_dst, uint8_t* dst_scale, uint32_t ld_dst_scale, uint32_t k, uint32_t n,
+                                    uint32_t batch, cmx_stream_t stream) {
+    return cmx::fp4_to_k_major(src, ld_src, src_scale, dst, ld_dst, dst_scale, ld_dst_scale, k, n, batch,
+                               static_cast<hipStream_t>(stream));
 }
 
 // the code part alone (INT8 weights stored [batch, k, n] -> [batch, n, k])
@@ -182,26 +311,27 @@ extern "C" int cmx_mx_gemm_ex(const uint8_t* a, const uint8_t* a_scale, const ui
                               int trans_b, void* workspace, cmx_stream_t stream) {
     using namespace cmx;
     if (m == 0 || n == 0) return CMX_OK;
-    CMX_REQUIRE(fmt_is_8bit(fmt), "layout normalisation covers the 8-bit element formats");
+    CMX_REQUIRE(fmt_has_layouts(fmt), "unknown element format");
     CMX_REQUIRE(k > 0 && k % 64 == 0, "k must be a positive multiple of 64");
-    const ExLayout L = ex_layout(m, n, k, trans_a, trans_b);
+    const ExLayout L = ex_layout(m, n, k, trans_a, trans_b, fmt);
     CMX_REQUIRE(L.total == 0 || (workspace && (reinterpret_cast<uintptr_t>(workspace) & 255u) == 0),
                 "workspace missing or not 256-byte aligned");
     uint8_t* ws = static_cast<uint8_t*>(workspace);
     hipStream_t s = static_cast<hipStream_t>(stream);
+    const uint32_t kbytes = fmt == CMX_FMT_E2M1 ? k / 2 : k;
     if (trans_a) {
-        int rc = to_k_major(a, m, a_scale, ws + L.a_codes, k, ws + L.a_scales, k / 32, k, m, 1, s);
+        int rc = normalise(a, a_scale, ws + L.a_codes, ws + L.a_scales, k, m, 1, fmt, s);
         if (rc != CMX_OK) return rc;
         a = ws + L.a_codes;
         a_scale = ws + L.a_scales;
     }
     if (!trans_b) {
-        int rc = to_k_major(b, n, b_scale, ws + L.b_codes, k, ws + L.b_scales, k / 32, k, n, 1, s);
+        int rc = normalise(b, b_scale, ws + L.b_codes, ws + L.b_scales, k, n, 1, fmt, s);
         if (rc != CMX_OK) return rc;
         b = ws + L.b_codes;
         b_scale = ws + L.b_scales;
     }
-    return cmx_mx_gemm(a, k, a_scale, k / 32, b, k, b_scale, k / 32, c, ldc, m, n, k, fmt, out_type, stream);
+    return cmx_mx_gemm(a, kbytes, a_scale, k / 32, b, kbytes, b_scale, k / 32, c, ldc, m, n, k, fmt, out_type, stream);
 }
 
 extern "C" size_t cmx_mx_gmm_ex_workspace_bytes(uint32_t groups, uint32_t n, uint32_t k, int trans_b) {
@@ -214,19 +344,21 @@ extern "C" int cmx_mx_gmm_ex(const uint8_t* a, const uint8_t* a_scale, const uin
                              uint32_t k, int fmt, int out_type, int trans_b, void* workspace, cmx_stream_t stream) {
     using namespace cmx;
     if (m_total == 0 || n == 0) return CMX_OK;
-    CMX_REQUIRE(fmt_is_8bit(fmt), "layout normalisation covers the 8-bit element formats");
+    CMX_REQUIRE(fmt_has_layouts(fmt), "unknown element format");
     CMX_REQUIRE(k > 0 && k % 64 == 0, "k must be a positive multiple of 64");
     CMX_REQUIRE(groups > 0 && workspace && (reinterpret_cast<uintptr_t>(workspace) & 255u) == 0,
                 "workspace missing or not 256-byte aligned");
     uint8_t* ws = static_cast<uint8_t*>(workspace);
     const size_t meta = round_up_sz(cmx_mx_gmm_workspace_bytes(groups), 256);
     if (!trans_b) {
-        const ExLayout L = ex_layout(0, (uint64_t)groups * n, k, 0, 0);
-        int rc = to_k_major(b, n, b_scale, ws + meta + L.b_codes, k, ws + meta + L.b_scales, k / 32, k, n, groups,
-                            static_cast<hipStream_t>(stream));
+        CMX_REQUIRE(fmt != CMX_FMT_E2M1 || n % 2 == 0, "FP4 weights stored [groups, k, n / 2] need an even n");
+        const ExLayout L = ex_layout(0, (uint64_t)groups * n, k, 0, 0, fmt);
+        int rc = normalise(b, b_scale, ws + meta + L.b_codes, ws + meta + L.b_scales, k, n, groups, fmt,
+                           static_cast<hipStream_t>(stream));
         if (rc != CMX_OK) return rc;
         b = ws + meta + L.b_codes;
         b_scale = ws + meta + L.b_scales;
     }
-    return cmx_mx_gmm(a, k, a_scale, k / 32, b, b_scale, c, ldc, group_sizes, groups, m_total, n, k, fmt, out_type, ws, stream);
+    const uint32_t kbytes = fmt == CMX_FMT_E2M1 ? k / 2 : k;
+    return cmx_mx_gmm(a, kbytes, a_scale, k / 32, b, b_scale, c, ldc, group_sizes, groups, m_total, n, k, fmt, out_type, ws, stream);
 }

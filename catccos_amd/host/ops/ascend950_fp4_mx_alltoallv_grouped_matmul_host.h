@@ -2,7 +2,9 @@
 // rows of each local expert, fp16 output.  With one rank the all-to-all is the identity: A's rows already
 // sit in expert order.  Host contract follows
 // examples/ascend950_fp4_mx_alltoallv_grouped_matmul/ascend950_fp4_mx_alltoallv_grouped_matmul_host.h:16-184.
-// B must be stored transposed per expert ([E, N, K/2] codes, [E, N, K/32] scales; transB = 1).
+// B comes in either orientation of the reference's generator (examples/utils/gen_data_fp4_mx_alltoallv_gmm.py:586-620):
+// [E, K, N/2] bytes with scales [E, K/64, N, 2] (transB = 0, the setting of the example's run.sh) or [E, N, K/2] with
+// [E, N, K/64, 2] (transB = 1); the first is rewritten K-contiguous in the workspace before the matmul.
 #ifndef ASCEND950_FP4_MX_ALLTOALLV_GROUPED_MATMUL_HOST_H
 #define ASCEND950_FP4_MX_ALLTOALLV_GROUPED_MATMUL_HOST_H
 
@@ -51,7 +53,10 @@ public:
         mxops::DeviceBufferToFile(params.ptrC, cBytes, mxops::RankFile(dataFile, "output", rankId, false));
     }
 
-    size_t GetWorkspaceSize(const CocTilingParams& t) override { return cmx_mx_gmm_workspace_bytes(t.expertNum / (t.epSize ? t.epSize : 1)); }
+    size_t GetWorkspaceSize(const CocTilingParams& t) override
+    {
+        return cmx_mx_gmm_ex_workspace_bytes(t.expertNum / (t.epSize ? t.epSize : 1), t.n, t.k, static_cast<int>(t.transB));
+    }
     CocCommType GetActualKernelType(const CocTilingParams&) override { return CocCommType::ASCEND950_FP4_MX_ALLTOALLV_GROUPED_MATMUL; }
 
     bool CheckCocTilingParams(uint32_t rankSize, const CocTilingParams& t) override
@@ -68,8 +73,8 @@ public:
         if (static_cast<int64_t>(t.commInterval) * t.m0 * t.k0 * kLoop >= maxPeerMemPerRank) {
             return false;
         }
-        if (t.transB != 1 || t.k % 64 != 0) {
-            std::cerr << "MXFP4 grouped matmul needs transposed weights ([E,N,K/2]) and K % 64 == 0" << std::endl;
+        if (t.transA != 0 || t.transB > 1 || t.k % 64 != 0 || (t.transB == 0 && t.n % 2 != 0)) {
+            std::cerr << "MXFP4 grouped matmul needs row-major A, transB 0 or 1, K % 64 == 0 (and an even N with transB = 0)" << std::endl;
             return false;
         }
         return true;
@@ -78,9 +83,9 @@ public:
     static int Launch(void* stream, const KernelParams& p, uint8_t* workspace, const CocTilingParams& t)
     {
         const uint32_t experts = t.expertNum / t.epSize;
-        return cmx_mx_gmm(p.ptrA, t.k / 2, p.customPtrs[0], t.k / 32, p.ptrB, p.customPtrs[1], p.ptrC, t.n,
-                          reinterpret_cast<const int32_t*>(p.customPtrs[3]), experts, t.m * t.rankSize, t.n, t.k, CMX_FMT_E2M1,
-                          CMX_OUT_FP16, workspace, stream);
+        return cmx_mx_gmm_ex(p.ptrA, p.customPtrs[0], p.ptrB, p.customPtrs[1], p.ptrC, t.n,
+                             reinterpret_cast<const int32_t*>(p.customPtrs[3]), experts, t.m * t.rankSize, t.n, t.k, CMX_FMT_E2M1,
+                             CMX_OUT_FP16, static_cast<int>(t.transB), workspace, stream);
     }
 };
 

@@ -24,9 +24,12 @@ void LaunchFfn(void* stream, uint32_t, uint64_t, KernelParams& p, uint8_t* ws, u
 {
     LaunchStatus() = Ascend950DispatchFFNCombineOperator::Launch(stream, p, p.ptrC, ws, symm, t);
 }
-void LaunchFp4Gmm(void* stream, uint32_t, uint64_t, KernelParams& p, uint8_t* ws, uint8_t*, CocTilingParams& t, uint32_t, uint32_t)
+void LaunchFp4Gmm(void* stream, uint32_t, uint64_t, KernelParams& p, uint8_t* ws, uint8_t*, CocTilingParams& t, uint32_t transA, uint32_t transB)
 {
-    LaunchStatus() = Ascend950Fp4MxAllToAllVGroupedMatmulOperator::Launch(stream, p, ws, t);
+    CocTilingParams tt = t;
+    tt.transA = transA;
+    tt.transB = transB;
+    LaunchStatus() = Ascend950Fp4MxAllToAllVGroupedMatmulOperator::Launch(stream, p, ws, tt);
 }
 void LaunchDgds(void* stream, uint32_t, uint64_t, KernelParams& p, uint8_t* ws, uint8_t*, CocTilingParams& t, uint32_t, uint32_t)
 {

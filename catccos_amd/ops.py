@@ -87,6 +87,20 @@ def mx_to_k_major(src, src_scale, k: int, n: int):
     return dst, dst_scale
 
 
+def mxfp4_to_k_major(src, src_scale, k: int, n: int):
+    """FP4: bytes [batch, k, ceil(n/2)] (pairs along n) with scales [batch, k/64, n, 2] -> bytes [batch, n, k/2], scales [batch, n, k/32]."""
+    _need_cuda(src, src_scale)
+    assert src.is_contiguous() and src_scale.is_contiguous()
+    batch = src.shape[0] if src.dim() == 3 else 1
+    shape = (batch, n) if src.dim() == 3 else (n,)
+    dst = torch.empty(shape + (k // 2,), dtype=torch.uint8, device=src.device)
+    dst_scale = torch.empty(shape + (k // 32,), dtype=torch.uint8, device=src.device)
+    lib = _lib.load()
+    _lib.check(lib.cmx_mxfp4_to_k_major(_p(src), (n + 1) // 2, _p(src_scale), _p(dst), k // 2, _p(dst_scale), k // 32, k, n, batch,
+                                        _stream()))
+    return dst, dst_scale
+
+
 def mx_gemm_ex(a, a_scale, b, b_scale, m: int, n: int, k: int, fmt: str = "E4M3", out: str = "bf16", trans_a: int = 0,
                trans_b: int = 1) -> torch.Tensor:
     """Dense operands in the reference's file layouts: a [m, k] (trans_a = 1: [k, m], scales [k/64, m, 2]);

@@ -152,6 +152,10 @@ int cmx_mx_gmm_swiglu_quant(const uint8_t* a, uint32_t lda, const uint8_t* a_sca
  * cmx_mx_to_k_major rewrites `batch` such operands (codes [batch, k, n] with row pitch ld_src, scales
  * [batch, k/64, n, 2] dense) as K-contiguous ones (codes [batch, n, k] with row pitch ld_dst, scales
  * [batch, n, k/32] with row pitch ld_dst_scale).  8-bit element formats; k a multiple of 64.
+ * cmx_mxfp4_to_k_major is the same for FP4, where two codes share a byte along the contiguous axis
+ * (examples/utils/gen_data_fp4_mx_alltoallv_gmm.py:522-545, 586-620): codes [batch, k, ceil(n/2)] bytes (pairs
+ * along n, even column in the low nibble) -> [batch, n, k/2] bytes (pairs along k); pitches in bytes.  The
+ * *_ex entry points take CMX_FMT_E2M1 as well (their workspace size functions give the 8-bit size, an upper bound).
  *
  * cmx_mx_gemm_ex / cmx_mx_gmm_ex are cmx_mx_gemm / cmx_mx_gmm for dense operands in either orientation
  * (trans_a = 1: A is [K, M]; trans_b = 0: B is [K, N] resp. [groups, K, N]); operands that are not K-contiguous
@@ -162,6 +166,9 @@ int cmx_mx_gmm_swiglu_quant(const uint8_t* a, uint32_t lda, const uint8_t* a_sca
 int cmx_mx_to_k_major(const uint8_t* src, uint32_t ld_src, const uint8_t* src_scale, uint8_t* dst, uint32_t ld_dst,
                       uint8_t* dst_scale, uint32_t ld_dst_scale, uint32_t k, uint32_t n, uint32_t batch,
                       cmx_stream_t stream);
+int cmx_mxfp4_to_k_major(const uint8_t* src, uint32_t ld_src, const uint8_t* src_scale, uint8_t* dst, uint32_t ld_dst,
+                         uint8_t* dst_scale, uint32_t ld_dst_scale, uint32_t k, uint32_t n, uint32_t batch,
+                         cmx_stream_t stream);
 size_t cmx_mx_gemm_ex_workspace_bytes(uint32_t m, uint32_t n, uint32_t k, int trans_a, int trans_b);
 int cmx_mx_gemm_ex(const uint8_t* a, const uint8_t* a_scale, const uint8_t* b, const uint8_t* b_scale, void* c,
                    uint32_t ldc, uint32_t m, uint32_t n, uint32_t k, int fmt, int out_type, int trans_a, int trans_b,

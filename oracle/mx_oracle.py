@@ -388,6 +388,21 @@ def from_file_layout(codes, scales, trans: bool):
     return np.ascontiguousarray(codes.T), np.ascontiguousarray(scales.reshape(k // 64, r, 2).transpose(1, 0, 2).reshape(r, k // 32))
 
 
+def to_file_layout_fp4(codes, scales, trans: bool):
+    """FP4 counterpart of :func:`to_file_layout` for un-packed codes [R, K]: the generator packs two codes per byte
+    along the LAST axis of whichever orientation it writes (matrix_fp32_to_fp4,
+    gen_data_fp4_mx_alltoallv_gmm.py:522-545; orientation and scale permutes :586-620).  trans False: bytes
+    [R, K/2] (pairs along K), scales [R, K/64, 2].  trans True: bytes [K, ceil(R/2)] (pairs along R), scales
+    [K/64, R, 2]."""
+    codes = np.asarray(codes)
+    scales = np.asarray(scales)
+    r, k = codes.shape
+    pairs = scales[:, :k // 32].reshape(r, k // 64, 2)
+    if not trans:
+        return pack_fp4(codes), np.ascontiguousarray(pairs)
+    return pack_fp4(np.ascontiguousarray(codes.T)), np.ascontiguousarray(pairs.transpose(1, 0, 2))
+
+
 def mx_gemm_bf16(*args, **kw) -> np.ndarray:
     """bf16 result (bit pattern) of :func:`mx_gemm_f32` (gen_data_moe.py:650)."""
     return f32_to_bf16_bits(mx_gemm_f32(*args, **kw))

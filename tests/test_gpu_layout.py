@@ -85,12 +85,60 @@ def test_gmm_ex_with_k_slow_weights():
     assert bad == 0, (bad, worst)
 
 
+@pytest.mark.parametrize("n,k", [(128, 128), (2, 64), (37, 192), (130, 320), (4096, 7168), (255, 64), (64, 1024)])
+def test_fp4_to_k_major_is_bit_exact(n, k):
+    from catccos_amd import ops
+    rng = np.random.default_rng(n * 3 + k)
+    codes = rng.integers(0, 16, size=(n, k), dtype=np.uint8)
+    scales = rng.integers(0, 256, size=(n, k // 32), dtype=np.uint8)
+    fb, fs = O.to_file_layout_fp4(codes, scales, True)
+    d, ds = ops.mxfp4_to_k_major(dev(fb), dev(fs), k, n)
+    assert np.array_equal(host(d), O.pack_fp4(codes))
+    assert np.array_equal(host(ds), scales)
+
+
+def test_fp4_batched_weights_and_grouped_matmul_ex():
+    from catccos_amd import ops
+    rng = np.random.default_rng(29)
+    counts = [40, 0, 129, 300]
+    n, k = 256, 512
+    m = sum(counts)
+    aq, asc = O.mx_quant(rng.uniform(-2, 2, (m, k)).astype(np.float32), "E2M1")
+    ws_ = [O.mx_quant(rng.uniform(-2, 2, (n, k)).astype(np.float32), "E2M1") for _ in counts]
+    wq, wsc = np.stack([q for q, _ in ws_]), np.stack([s_ for _, s_ in ws_])
+    fw = np.stack([O.to_file_layout_fp4(wq[i], wsc[i], True)[0] for i in range(len(counts))])
+    fws = np.stack([O.to_file_layout_fp4(wq[i], wsc[i], True)[1] for i in range(len(counts))])
+    d, ds = ops.mxfp4_to_k_major(dev(fw), dev(fws), k, n)
+    assert np.array_equal(host(d), np.stack([O.pack_fp4(w) for w in wq])) and np.array_equal(host(ds), wsc)
+    gs = dev(np.array(counts, dtype=np.int32))
+    c0 = ops.mx_gmm_ex(dev(O.pack_fp4(aq)), dev(asc), dev(fw), dev(fws), gs, n, k, "E2M1", "fp16", trans_b=0)
+    c1 = ops.mx_gmm(dev(O.pack_fp4(aq)), dev(asc), dev(O.pack_fp4(wq)), dev(wsc), gs, k, "E2M1", "fp16")
+    assert np.array_equal(host(c0), host(c1))
+    gold = O.mx_gmm_f32(aq, asc, wq, wsc, counts, "E2M1", "E2M1")
+    assert np.allclose(host(c0).astype(np.float64), gold, rtol=2e-3, atol=5e-2)
+
+
+def test_fp4_gemm_ex_orientations():
+    from catccos_amd import ops
+    rng = np.random.default_rng(30)
+    m, n, k = 130, 300, 640
+    aq, asc = O.mx_quant(rng.uniform(-2, 2, (m, k)).astype(np.float32), "E2M1")
+    bq, bsc = O.mx_quant(rng.uniform(-2, 2, (n, k)).astype(np.float32), "E2M1")
+    ref = ops.mx_gemm(dev(O.pack_fp4(aq)), dev(asc), dev(O.pack_fp4(bq)), dev(bsc), k, "E2M1", "fp32")
+    for trans_a, trans_b in [(0, 0), (1, 1), (1, 0)]:
+        fa, fas = O.to_file_layout_fp4(aq, asc, bool(trans_a))
+        fb, fbs = O.to_file_layout_fp4(bq, bsc, not trans_b)
+        c = ops.mx_gemm_ex(dev(fa), dev(fas), dev(fb), dev(fbs), m, n, k, "E2M1", "fp32", trans_a, trans_b)
+        assert np.array_equal(host(c), host(ref)), (trans_a, trans_b)
+    assert np.allclose(host(ref), O.mx_gemm_f32(aq, asc, bq, bsc, "E2M1", "E2M1"), rtol=1e-5, atol=1e-3)
+
+
 def test_ex_entry_points_reject_what_they_do_not_cover():
     from catccos_amd import _lib
     lib = _lib.load()
     z = torch.zeros(1 << 16, dtype=torch.uint8, device="cuda")
     p = z.data_ptr()
-    assert lib.cmx_mx_gemm_ex(p, p, p, p, p, 64, 64, 64, 64, 2, 0, 0, 0, p, None) == -1      # FP4
+    assert lib.cmx_mx_gemm_ex(p, p, p, p, p, 64, 64, 64, 64, 3, 0, 0, 0, p, None) == -1      # E1M2 has no matmul
     assert lib.cmx_mx_gemm_ex(p, p, p, p, p, 64, 64, 64, 96, 0, 0, 0, 0, p, None) == -1      # k % 64
     assert lib.cmx_mx_gemm_ex(p, p, p, p, p, 64, 64, 64, 64, 0, 0, 0, 0, None, None) == -1   # workspace missing
     assert lib.cmx_mx_gemm_ex_workspace_bytes(64, 64, 64, 0, 1) == 0

@@ -115,6 +115,31 @@ def test_driver_mxfp8_matmul_operand_orientations(host_bin, tmp_path, trans_a, t
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("trans_b", [0, 1])
+def test_driver_fp4_grouped_matmul(host_bin, tmp_path, trans_b):
+    """The reference's file names and both weight orientations of its generator (transB = 0 is its run.sh default:
+    examples/ascend950_fp4_mx_alltoallv_grouped_matmul/scripts/run.sh:16-17)."""
+    experts, n, k = 4, 192, 256
+    counts = np.array([40, 0, 70, 18], dtype=np.int32)
+    m = int(counts.sum())
+    rng = np.random.default_rng(19)
+    aq, asc = O.mx_quant(rng.uniform(-2, 2, (m, k)).astype(np.float32), "E2M1")
+    ws_ = [O.mx_quant(rng.uniform(-2, 2, (n, k)).astype(np.float32), "E2M1") for _ in range(experts)]
+    wq, wsc = np.stack([q for q, _ in ws_]), np.stack([s_ for _, s_ in ws_])
+    fb = np.stack([O.to_file_layout_fp4(wq[i], wsc[i], not trans_b)[0] for i in range(experts)])
+    fbs = np.stack([O.to_file_layout_fp4(wq[i], wsc[i], not trans_b)[1] for i in range(experts)])
+    fa, fas = O.to_file_layout_fp4(aq, asc, False)
+    for stem, arr in (("input_a", fa), ("input_a_scale", fas), ("input_b", fb), ("input_b_scale", fbs),
+                      ("local_tokens_per_expert", counts), ("global_tokens_per_local_expert", counts)):
+        _write(tmp_path / f"{stem}_0.bin", arr)
+    r = _run(host_bin, "a5fp4mxatavgmm", m, k, n, "--experts", experts, "--data", tmp_path, "--transb", trans_b, "--poison")
+    assert r.returncode == 0, r.stdout + r.stderr
+    got = np.fromfile(tmp_path / "output_0.bin", dtype=np.float16).reshape(m, n).astype(np.float64)
+    gold = O.mx_gmm_f32(aq, asc, wq, wsc, counts, "E2M1", "E2M1")
+    assert np.allclose(got, gold, rtol=2e-3, atol=5e-2)
+
+
+@pytest.mark.gpu
 def test_driver_int8_dispatch_gmm_dequant_swiglu(host_bin, tmp_path):
     """The reference operator's own arithmetic and file names (examples/dispatch_gmm_dequant_swiglu/
     dispatch_gmm_dequant_swiglu_host.h:31-73): a_gm bf16 [m, k], b_gm int8 [E, k, n], scale_gm 64-bit words,

@@ -251,3 +251,23 @@ def test_file_layouts_of_operands_by_explicit_indexing():
     for trans in (False, True):
         c2, s2 = O.from_file_layout(*O.to_file_layout(codes, scales, trans), trans)
         assert np.array_equal(c2, codes) and np.array_equal(s2, scales[:, :k // 32])
+
+
+def test_fp4_file_layouts_by_explicit_indexing():
+    """FP4 bytes of the K-slow orientation: code (r, k) sits in byte [k, r // 2], low nibble for even r
+    (gen_data_fp4_mx_alltoallv_gmm.py:522-545 applied to the transposed matrix, :586-620)."""
+    rng = np.random.default_rng(22)
+    r, k = 7, 128
+    codes = rng.integers(0, 16, size=(r, k), dtype=np.uint8)
+    scales = rng.integers(100, 140, size=(r, k // 32), dtype=np.uint8)
+    fb, fs = O.to_file_layout_fp4(codes, scales, True)
+    assert fb.shape == (k, (r + 1) // 2) and fs.shape == (k // 64, r, 2)
+    for i in range(r):
+        for kk in range(k):
+            byte = int(fb[kk, i // 2])
+            assert ((byte >> 4) if i % 2 else (byte & 15)) == codes[i, kk]
+            kb = kk // 32
+            assert fs[kb // 2, i, kb % 2] == scales[i, kb]
+    assert np.all(fb[:, -1] >> 4 == 0)                       # the odd row count leaves the last high nibble empty
+    nb, ns = O.to_file_layout_fp4(codes, scales, False)
+    assert np.array_equal(nb, O.pack_fp4(codes)) and np.array_equal(ns.reshape(r, -1), scales)
