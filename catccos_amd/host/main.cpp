@@ -2,7 +2,8 @@
 //
 //   catccos_mx_run <operator> M K N [options]
 //     <operator>    registry name ("Ascend950DispatchFFNCombine", ...) or short name ("a5moe", "mxqtag",
-//                   "a5mxfp8mmrs", "a5fp4mxatavgmm", "dgds")
+//                   "a5mxfp8mmrs", "a5fp4mxatavgmm", "dgds", "a5fp8mxagmm", "a5fp4mxagmm", "a5mxfp8mmata", "a5fp4mmrs",
+//                   "a5fp8mxatavgmm", "a5fp8gmmata", "a5fp4gmmata")
 //     --experts E   local experts (MoE operators; default 4)      --topk T     routes per token (default 4)
 //     --data DIR    directory with the operator's input .bin files; outputs are written there too
 //                   (without it inputs are defaults / zeros and nothing is written)
@@ -27,6 +28,7 @@
 #include "launch_map.h"
 #include "ops/ascend950_mxfp8_matmul_reduce_scatter_host.h"
 #include "ops/dispatch_gmm_dequant_swiglu_host.h"
+#include "ops/mx_matmul_family_host.h"
 #include "ops/mx_quant_allgather_host.h"
 
 namespace {
@@ -113,6 +115,12 @@ int Run(int argc, char** argv)
     MxQuantAllGatherOperator::ElementFormat() = fmt;
     DispatchGmmDequantSwigluOperator::Arithmetic() =
         o.arith == "int8" ? DispatchGmmDequantSwigluOperator::kInt8 : DispatchGmmDequantSwigluOperator::kMx;
+    if (fmt == CMX_FMT_E4M3 || fmt == CMX_FMT_E5M2) {
+        Ascend950Fp8MxAllGatherMatmulOperator::Fp8Format() = fmt;
+        Ascend950MxFp8MatmulAllToAllOperator::Fp8Format() = fmt;
+        Ascend950Fp8MxAllToAllVGroupedMatmulOperator::Fp8Format() = fmt;
+        Ascend950Fp8MxGroupedMatmulAllToAllVOperator::Fp8Format() = fmt;
+    }
     const bool fp4 = fmt == CMX_FMT_E2M1 || fmt == CMX_FMT_E1M2;
     MxQuantAllGatherOperator::RoundMode() = fp4 ? CMX_ROUND_LUT : CMX_ROUND_RNE;
     Ascend950MxFp8MatmulReduceScatterOperator::ElementFormat() = fp4 ? CMX_FMT_E4M3 : fmt;
@@ -142,8 +150,9 @@ int Run(int argc, char** argv)
         std::cerr << "Invalid CocTilingParams" << std::endl;
         return -1;
     }
-    const CocDataType dtype = type == ASCEND950_FP4_MX_ALLTOALLV_GROUPED_MATMUL ? FP16 : BF16;
-    KernelFuncPtr launch = GetKernelFunc(op->GetActualKernelType(tiling), dtype);
+    // the operators with fp16 output are registered under FP16, the others under BF16
+    KernelFuncPtr launch = GetKernelFunc(op->GetActualKernelType(tiling), BF16);
+    if (!launch) launch = GetKernelFunc(op->GetActualKernelType(tiling), FP16);
     if (!launch) {
         std::cerr << "[ERROR] no launch entry for " << opName << std::endl;
         return 1;

@@ -5,6 +5,7 @@
 #include "ascend950_fp4_mx_alltoallv_grouped_matmul_host.h"
 #include "ascend950_mxfp8_matmul_reduce_scatter_host.h"
 #include "dispatch_gmm_dequant_swiglu_host.h"
+#include "mx_matmul_family_host.h"
 #include "mx_quant_allgather_host.h"
 
 namespace {
@@ -36,6 +37,15 @@ void LaunchDgds(void* stream, uint32_t, uint64_t, KernelParams& p, uint8_t* ws, 
     LaunchStatus() = DispatchGmmDequantSwigluOperator::Launch(stream, p, ws, t);
 }
 
+template <class Op>
+void LaunchFamily(void* stream, uint32_t, uint64_t, KernelParams& p, uint8_t* ws, uint8_t*, CocTilingParams& t, uint32_t transA, uint32_t transB)
+{
+    CocTilingParams tt = t;
+    tt.transA = transA;
+    tt.transB = transB;
+    LaunchStatus() = Op::Launch(stream, p, ws, tt);
+}
+
 }  // namespace
 
 std::map<uint32_t, KernelFuncPtr>& LaunchMap()
@@ -47,6 +57,13 @@ std::map<uint32_t, KernelFuncPtr>& LaunchMap()
         {LaunchKey(ASCEND950_DISPATCH_FFN_COMBINE, BF16), LaunchFfn},
         {LaunchKey(ASCEND950_FP4_MX_ALLTOALLV_GROUPED_MATMUL, FP16), LaunchFp4Gmm},
         {LaunchKey(DISPATCH_GMM_DEQUANT_SWIGLU, BF16), LaunchDgds},
+        {LaunchKey(ASCEND950_FP8_MX_ALLGATHER_MATMUL, FP16), LaunchFamily<Ascend950Fp8MxAllGatherMatmulOperator>},
+        {LaunchKey(ASCEND950_FP4_MX_ALLGATHER_MATMUL, FP16), LaunchFamily<Ascend950Fp4MxAllGatherMatmulOperator>},
+        {LaunchKey(ASCEND950_MXFP8_MATMUL_ALLTOALL, FP16), LaunchFamily<Ascend950MxFp8MatmulAllToAllOperator>},
+        {LaunchKey(ASCEND950_FP4_MX_MATMUL_REDUCE_SCATTER, FP16), LaunchFamily<Ascend950Fp4MxMatmulReduceScatterOperator>},
+        {LaunchKey(ASCEND950_FP8_MX_ALLTOALLV_GROUPED_MATMUL, FP16), LaunchFamily<Ascend950Fp8MxAllToAllVGroupedMatmulOperator>},
+        {LaunchKey(ASCEND950_FP8_MX_GROUPED_MATMUL_ALLTOALLV, FP16), LaunchFamily<Ascend950Fp8MxGroupedMatmulAllToAllVOperator>},
+        {LaunchKey(ASCEND950_FP4_MX_GROUPED_MATMUL_ALLTOALLV, FP16), LaunchFamily<Ascend950Fp4MxGroupedMatmulAllToAllVOperator>},
     };
     return table;
 }

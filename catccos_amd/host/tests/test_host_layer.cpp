@@ -30,10 +30,13 @@ int main()
     EXPECT(Ub::Fits(1, 14336, 8, 48) && !Ub::Fits(1, 14592, 8, 48) && !Ub::Fits(1, 2048, 8, 0));
     EXPECT(Ub::Fits(28800, 2048, 46, 48) && !Ub::Fits(28800, 2048, 47, 48) && Ub::Fits(1, 7168, 6, 48));
 
-    // registry: the five operators register themselves under the reference's names
+    // registry: the operators register themselves under the reference's names
     auto& reg = OperatorRegistry::Instance();
     for (const char* name : {"MxQuantAllGather", "Ascend950MxFp8MatmulReduceScatter", "Ascend950DispatchFFNCombine",
-                             "Ascend950Fp4MxAllToAllVGroupedMatmul", "DispatchGmmDequantSwiglu"}) {
+                             "Ascend950Fp4MxAllToAllVGroupedMatmul", "DispatchGmmDequantSwiglu", "Ascend950Fp8MxAllGatherMatmul",
+                             "Ascend950Fp4MxAllGatherMatmul", "Ascend950MxFp8MatmulAllToAll", "Ascend950Fp4MxMatmulReduceScatter",
+                             "Ascend950Fp8MxAllToAllVGroupedMatmul", "Ascend950Fp8MxGroupedMatmulAllToAllV",
+                             "Ascend950Fp4MxGroupedMatmulAllToAllV"}) {
         EXPECT(reg.CreateOperator(name) != nullptr);
     }
     EXPECT(reg.CreateOperator("NoSuchOperator") == nullptr);

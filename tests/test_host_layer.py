@@ -139,6 +139,52 @@ def test_driver_fp4_grouped_matmul(host_bin, tmp_path, trans_b):
     assert np.allclose(got, gold, rtol=2e-3, atol=5e-2)
 
 
+FAMILY = [   # short name, fp4, grouped, file name style, output file
+    ("a5fp8mxagmm", False, False, "input", "output_0.bin"),
+    ("a5fp4mxagmm", True, False, "input", "output_0.bin"),
+    ("a5mxfp8mmata", False, False, "rank", "output_0.bin"),
+    ("a5fp4mmrs", True, False, "rank", "output.bin"),
+    ("a5fp8mxatavgmm", False, True, "input", "output_0.bin"),
+    ("a5fp8gmmata", False, True, "gm", "output_0.bin"),
+    ("a5fp4gmmata", True, True, "gm", "output_0.bin"),
+]
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("short,fp4,grouped,style,outfile", FAMILY)
+def test_driver_mx_matmul_family(host_bin, tmp_path, short, fp4, grouped, style, outfile):
+    """The other MX matmul operators of the reference under their own names, file names and default orientation
+    (transB = 0: weights [K, N] with scales [K/64, N, 2]); fp16 output."""
+    fmt = "E2M1" if fp4 else "E4M3"
+    experts, n, k = (4 if grouped else 1), 192, 256
+    counts = np.array([40, 0, 70, 18], dtype=np.int32) if grouped else np.array([96], dtype=np.int32)
+    m = int(counts.sum())
+    rng = np.random.default_rng(len(short) + 7 * fp4)
+    gen = (lambda r: rng.uniform(-2, 2, (r, k)).astype(np.float32)) if fp4 else \
+          (lambda r: O.bf16_round(rng.standard_normal((r, k)).astype(np.float32)))
+    aq, asc = O.mx_quant(gen(m), fmt)
+    ws_ = [O.mx_quant(gen(n), fmt) for _ in range(experts)]
+    wq, wsc = np.stack([q for q, _ in ws_]), np.stack([s_ for _, s_ in ws_])
+    lay = O.to_file_layout_fp4 if fp4 else O.to_file_layout
+    fb = np.stack([lay(wq[i], wsc[i], True)[0] for i in range(experts)])
+    fbs = np.stack([lay(wq[i], wsc[i], True)[1] for i in range(experts)])
+    fa, fas = lay(aq, asc, False)
+    name = {"input": lambda w: f"input_{w}_0.bin", "rank": lambda w: f"rank_0_{w}.bin",
+            "gm": lambda w: (f"{w}_gm_0.bin" if w in ("a", "b") else f"{w}_0.bin")}[style]
+    for what, arr in (("a", fa), ("b", fb), ("a_scale", fas), ("b_scale", fbs)):
+        _write(tmp_path / name(what), arr)
+    args = [short, m, k, n, "--data", tmp_path, "--transb", 0, "--poison"]
+    if grouped:
+        _write(tmp_path / "local_tokens_per_expert_0.bin", counts)
+        _write(tmp_path / "global_tokens_per_local_expert_0.bin", counts)
+        args += ["--experts", experts]
+    r = _run(host_bin, *args)
+    assert r.returncode == 0, r.stdout + r.stderr
+    got = np.fromfile(tmp_path / outfile, dtype=np.float16).reshape(m, n).astype(np.float64)
+    gold = O.mx_gmm_f32(aq, asc, wq, wsc, counts, fmt, fmt)
+    assert np.allclose(got, gold, rtol=2e-3, atol=5e-2)
+
+
 @pytest.mark.gpu
 def test_driver_int8_dispatch_gmm_dequant_swiglu(host_bin, tmp_path):
     """The reference operator's own arithmetic and file names (examples/dispatch_gmm_dequant_swiglu/
