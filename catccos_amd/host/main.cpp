@@ -118,6 +118,7 @@ int Run(int argc, char** argv)
     if (fmt == CMX_FMT_E4M3 || fmt == CMX_FMT_E5M2) {
         Ascend950Fp8MxAllGatherMatmulOperator::Fp8Format() = fmt;
         Ascend950MxFp8MatmulAllToAllOperator::Fp8Format() = fmt;
+        Ascend950MxFp8AllToAllMatmulSplitKUrmaOperator::Fp8Format() = fmt;
         Ascend950Fp8MxAllToAllVGroupedMatmulOperator::Fp8Format() = fmt;
         Ascend950Fp8MxGroupedMatmulAllToAllVOperator::Fp8Format() = fmt;
     }

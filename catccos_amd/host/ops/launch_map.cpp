@@ -60,6 +60,7 @@ std::map<uint32_t, KernelFuncPtr>& LaunchMap()
         {LaunchKey(ASCEND950_FP8_MX_ALLGATHER_MATMUL, FP16), LaunchFamily<Ascend950Fp8MxAllGatherMatmulOperator>},
         {LaunchKey(ASCEND950_FP4_MX_ALLGATHER_MATMUL, FP16), LaunchFamily<Ascend950Fp4MxAllGatherMatmulOperator>},
         {LaunchKey(ASCEND950_MXFP8_MATMUL_ALLTOALL, FP16), LaunchFamily<Ascend950MxFp8MatmulAllToAllOperator>},
+        {LaunchKey(ASCEND950_MXFP8_ALLTOALL_MATMUL_SPLIT_K_URMA, FP16), LaunchFamily<Ascend950MxFp8AllToAllMatmulSplitKUrmaOperator>},
         {LaunchKey(ASCEND950_FP4_MX_MATMUL_REDUCE_SCATTER, FP16), LaunchFamily<Ascend950Fp4MxMatmulReduceScatterOperator>},
         {LaunchKey(ASCEND950_FP8_MX_ALLTOALLV_GROUPED_MATMUL, FP16), LaunchFamily<Ascend950Fp8MxAllToAllVGroupedMatmulOperator>},
         {LaunchKey(ASCEND950_FP8_MX_GROUPED_MATMUL_ALLTOALLV, FP16), LaunchFamily<Ascend950Fp8MxGroupedMatmulAllToAllVOperator>},

@@ -6,6 +6,8 @@
 //   Ascend950Fp4MxAllGatherMatmul         examples/ascend950_fp4_mx_allgather_matmul/..._host.h                 dense   FP4
 //   Ascend950MxFp8MatmulAllToAll          examples/ascend950_mxfp8_matmul_alltoall/..._host.h:28-125            dense   FP8
 //   Ascend950Fp4MxMatmulReduceScatter     examples/ascend950_fp4_mx_matmul_reduce_scatter/..._host.h:20-110     dense   FP4
+//   Ascend950MxFp8AllToAllMatmulSplitKUrma examples/ascend950_mxfp8_alltoall_matmul_split_k_urma/..._host.h:30-125 dense  FP8
+//                                         (K is split over the ranks there: with one rank fullK = k, chunkM = m)
 //   Ascend950Fp8MxAllToAllVGroupedMatmul  examples/ascend950_fp8_mx_alltoallv_grouped_matmul/..._host.h         grouped FP8
 //   Ascend950Fp8MxGroupedMatmulAllToAllV  examples/ascend950_fp8_mx_grouped_matmul_alltoallv/..._host.h:18-180  grouped FP8
 //   Ascend950Fp4MxGroupedMatmulAllToAllV  examples/ascend950_fp4_mx_grouped_matmul_alltoallv/..._host.h         grouped FP4
@@ -132,6 +134,7 @@ public:
 class Ascend950Fp8MxAllGatherMatmulOperator : public mxops::MxMatmulFamilyOperator<ASCEND950_FP8_MX_ALLGATHER_MATMUL, false, false, mxops::FileNames::kInputA, mxops::OutputFile::kPerRank> {};
 class Ascend950Fp4MxAllGatherMatmulOperator : public mxops::MxMatmulFamilyOperator<ASCEND950_FP4_MX_ALLGATHER_MATMUL, true, false, mxops::FileNames::kInputA, mxops::OutputFile::kPerRank> {};
 class Ascend950MxFp8MatmulAllToAllOperator : public mxops::MxMatmulFamilyOperator<ASCEND950_MXFP8_MATMUL_ALLTOALL, false, false, mxops::FileNames::kRankA, mxops::OutputFile::kPerRank> {};
+class Ascend950MxFp8AllToAllMatmulSplitKUrmaOperator : public mxops::MxMatmulFamilyOperator<ASCEND950_MXFP8_ALLTOALL_MATMUL_SPLIT_K_URMA, false, false, mxops::FileNames::kInputA, mxops::OutputFile::kPerRank> {};
 class Ascend950Fp4MxMatmulReduceScatterOperator : public mxops::MxMatmulFamilyOperator<ASCEND950_FP4_MX_MATMUL_REDUCE_SCATTER, true, false, mxops::FileNames::kRankA, mxops::OutputFile::kShared> {};
 class Ascend950Fp8MxAllToAllVGroupedMatmulOperator : public mxops::MxMatmulFamilyOperator<ASCEND950_FP8_MX_ALLTOALLV_GROUPED_MATMUL, false, true, mxops::FileNames::kInputA, mxops::OutputFile::kPerRank> {};
 class Ascend950Fp8MxGroupedMatmulAllToAllVOperator : public mxops::MxMatmulFamilyOperator<ASCEND950_FP8_MX_GROUPED_MATMUL_ALLTOALLV, false, true, mxops::FileNames::kAGm, mxops::OutputFile::kPerRank> {};
@@ -140,6 +143,7 @@ class Ascend950Fp4MxGroupedMatmulAllToAllVOperator : public mxops::MxMatmulFamil
 REGISTER_OPERATOR("Ascend950Fp8MxAllGatherMatmul", Ascend950Fp8MxAllGatherMatmulOperator);
 REGISTER_OPERATOR("Ascend950Fp4MxAllGatherMatmul", Ascend950Fp4MxAllGatherMatmulOperator);
 REGISTER_OPERATOR("Ascend950MxFp8MatmulAllToAll", Ascend950MxFp8MatmulAllToAllOperator);
+REGISTER_OPERATOR("Ascend950MxFp8AllToAllMatmulSplitKUrma", Ascend950MxFp8AllToAllMatmulSplitKUrmaOperator);
 REGISTER_OPERATOR("Ascend950Fp4MxMatmulReduceScatter", Ascend950Fp4MxMatmulReduceScatterOperator);
 REGISTER_OPERATOR("Ascend950Fp8MxAllToAllVGroupedMatmul", Ascend950Fp8MxAllToAllVGroupedMatmulOperator);
 REGISTER_OPERATOR("Ascend950Fp8MxGroupedMatmulAllToAllV", Ascend950Fp8MxGroupedMatmulAllToAllVOperator);

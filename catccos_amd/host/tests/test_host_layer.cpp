@@ -36,7 +36,7 @@ int main()
                              "Ascend950Fp4MxAllToAllVGroupedMatmul", "DispatchGmmDequantSwiglu", "Ascend950Fp8MxAllGatherMatmul",
                              "Ascend950Fp4MxAllGatherMatmul", "Ascend950MxFp8MatmulAllToAll", "Ascend950Fp4MxMatmulReduceScatter",
                              "Ascend950Fp8MxAllToAllVGroupedMatmul", "Ascend950Fp8MxGroupedMatmulAllToAllV",
-                             "Ascend950Fp4MxGroupedMatmulAllToAllV"}) {
+                             "Ascend950Fp4MxGroupedMatmulAllToAllV", "Ascend950MxFp8AllToAllMatmulSplitKUrma"}) {
         EXPECT(reg.CreateOperator(name) != nullptr);
     }
     EXPECT(reg.CreateOperator("NoSuchOperator") == nullptr);

@@ -144,6 +144,7 @@ FAMILY = [   # short name, fp4, grouped, file name style, output file
     ("a5fp4mxagmm", True, False, "input", "output_0.bin"),
     ("a5mxfp8mmata", False, False, "rank", "output_0.bin"),
     ("a5fp4mmrs", True, False, "rank", "output.bin"),
+    ("a5mxfp8atammsplitkurma", False, False, "input", "output_0.bin"),
     ("a5fp8mxatavgmm", False, True, "input", "output_0.bin"),
     ("a5fp8gmmata", False, True, "gm", "output_0.bin"),
     ("a5fp4gmmata", True, True, "gm", "output_0.bin"),
