@@ -835,6 +835,7 @@ __global__ __launch_bounds__(64 * WW * WM) void mx_gemm_dl_kernel(const GemmPara
 }
 
 #include "mx_gemm_pipe.h"
+#include "mx_gemm_pipe_fp4.h"
 
 // Row offsets and m-tile prefix of the groups (one workgroup of 256 threads): each thread owns a contiguous run of
 // groups; the 256 partial sums are scanned in LDS, first for the rows, then for the m-tiles.
@@ -993,6 +994,19 @@ int launch_gemm_pipe(const GemmParams& p, uint32_t max_m_tiles, hipStream_t s) {
     return CMX_OK;
 }
 
+template <int EPI, int WW, int WM>
+int launch_gemm_pipe_fp4(const GemmParams& p, uint32_t max_m_tiles, hipStream_t s) {
+    constexpr size_t smem = 2 * 512 * kSlabBytes + 2 * 512 * 16;     // tile ring, ring of two scale blocks
+    auto kfn = mx_gemm_pipe_fp4_kernel<EPI, WW, WM>;
+    static PerDeviceFlag lds_allowed;
+    if (int rc = allow_dynamic_lds(kfn, smem, lds_allowed); rc != CMX_OK) return rc;
+    const uint64_t tiles = (uint64_t)max_m_tiles * p.w_tiles;
+    CMX_REQUIRE(tiles > 0 && tiles < (1ull << 31), "tile count out of range");
+    hipLaunchKernelGGL(kfn, dim3((uint32_t)tiles), dim3(256), smem, s, p);
+    CMX_LAUNCH_CHECK();
+    return CMX_OK;
+}
+
 bool g_disable_dl = false;   // tuning/test hook: force the register-staged kernels
 
 template <int FMT, int TW, int TM, int WW, int WM, int EPI>
@@ -1018,14 +1032,16 @@ TileChoice g_force_tile = {0, 0, 0};   // test/tuning hook: tw == 0 -> heuristic
 // from the LDS per slab and is the faster one on full tiles; grouped problems whose groups average less
 // than two tiles of rows take 4 x 1, where every wavefront shares in whatever rows a ragged tile has
 // (measured: 16 groups of ~2048 rows 891 vs 918 us in favour of 2 x 2, 256 groups of ~256 rows 4.33 vs
-// 4.38 ms in favour of 4 x 1).  FP4 takes the eight-wavefront streaming kernel.
+// 4.38 ms in favour of 4 x 1).  FP4 has its own hand-scheduled kernel in the same two layouts (K a multiple of 512
+// elements; 16 groups of ~2048 rows at K = 7168, N = 4096: 2 x 2 635 us, 4 x 1 700 us, the eight-wavefront
+// streaming kernel, which takes every other FP4 problem, 750 us).
 TileChoice choose_tile(uint32_t m_hint, uint32_t n, int fmt, bool grouped) {
     if (g_force_tile.tw) return g_force_tile;
     // short problems stream their weights once: the three-slot 256 x 128 kernel keeps two slabs in flight
     if (m_hint <= 128 && fmt != CMX_FMT_E2M1) return {256, 128, 5};
     if (m_hint <= 64) return {256, 64, 4};
     if (m_hint <= 128) return {256, 128, 8};
-    return {256, 256, fmt == CMX_FMT_E2M1 ? 8 : (grouped && m_hint < 512 ? 5 : 4)};
+    return {256, 256, grouped && m_hint < 512 ? 5 : 4};
 }
 
 // Eight-wavefront shapes exist only as streaming kernels; when a problem is not eligible for
@@ -1046,6 +1062,13 @@ int launch_tile(const GemmParams& p, int waves, uint32_t max_m_tiles, hipStream_
             if (lean) return launch_gemm_pipe<FMT, kLean, 256, 2, 2, 2>(p, max_m_tiles, s);
             if (waves == 4) return launch_gemm_pipe<FMT, EPI, 256, 2, 2, 2>(p, max_m_tiles, s);
             return launch_gemm_pipe<FMT, EPI, 256, 4, 1, 2>(p, max_m_tiles, s);
+        }
+    }
+    if constexpr (TW == 256 && TM == 256 && FMT == CMX_FMT_E2M1) {
+        // hand-scheduled FP4 kernel: whole two-slab scale blocks (K a multiple of 512 elements), 16-byte aligned scale rows
+        if ((waves == 4 || waves == 5) && stream_ok && p.scale_vec16 && p.kbytes % (2 * kSlabBytes) == 0) {
+            if (waves == 4) return launch_gemm_pipe_fp4<EPI, 2, 2>(p, max_m_tiles, s);
+            return launch_gemm_pipe_fp4<EPI, 4, 1>(p, max_m_tiles, s);
         }
     }
     if constexpr (TW == 256 && TM == 128 && FMT != CMX_FMT_E2M1) {

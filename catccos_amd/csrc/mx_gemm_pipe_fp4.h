@@ -1,0 +1,309 @@
+// Hand-scheduled 256 x 256 block-scaled matmul kernel for MXFP4 (E2M1, two codes per byte), included by
+// mx_gemm.hip after mx_gemm_pipe.h, whose helpers and conventions it shares.
+//
+// A 128-byte K slab holds 256 FP4 elements = four MFMA steps of 64 K; a lane's fragment of one step is a
+// single 16-byte run (the 32-element MX block of its half-wave), and a slab carries two scale dwords per
+// row.  As in the 8-bit two-slot kernels the scales arrive 16 bytes per row at a time -- here the scales of two
+// slabs -- into a ring of two such blocks, [block][row][4 dwords].  An FP4 MFMA takes 8 passes (32 clocks), so a slab is again 64 x 32 = 2048 MFMA clocks per wavefront
+// for the same 64 KiB of loads as in the 8-bit kernel.  Four wavefronts in a 2 x 2 grid, 16 accumulator
+// tiles in AGPRs, two fragment sets of 8 x 4 VGPRs.  Per slab s (ring slot s%2):
+//   step 0, 1: 16 MFMAs each; behind the first 8 the 8 reads of the next step's fragments (same slot);
+//   step 2:    likewise (reads of step 3); after MFMA 9 those have landed and the slot is never read again:
+//              barrier, then the first 6 tile loads of slab s+2 behind the remaining MFMAs; the step ends with
+//              the wait for the own loads of slab s+1 and the barrier that publishes it;
+//   step 3:    the other 10 tile loads of slab s+2 (and, every second slab, the next scale block), the reads of
+//              step 0 of slab s+1 from the other slot, its 16 scale dwords and their per-half-wave byte shift.
+#pragma once
+
+template <int SEL, int BIT>
+__device__ __forceinline__ void mfma_acc_fp4(v16f& acc, const v4i& w, const v4i& a, uint32_t sw, uint32_t sa, uint32_t live) {
+    static_assert(SEL == 0 || SEL == 2, "scale byte pair");
+    live = __builtin_amdgcn_readfirstlane(live);
+    if constexpr (BIT < 0) {
+        if constexpr (SEL == 0)
+            asm volatile("v_mfma_scale_f32_32x32x64_f8f6f4 %0, %1, %2, %0, %3, %4 op_sel_hi:[0,0,0] cbsz:4 blgp:4"
+                         : "+a"(acc) : "v"(w), "v"(a), "v"(sw), "v"(sa));
+        else
+            asm volatile("v_mfma_scale_f32_32x32x64_f8f6f4 %0, %1, %2, %0, %3, %4 op_sel_hi:[1,1,0] cbsz:4 blgp:4"
+                         : "+a"(acc) : "v"(w), "v"(a), "v"(sw), "v"(sa));
+    } else {
+        if constexpr (SEL == 0)
+            asm volatile("s_bitcmp1_b32 %5, %6\n\ts_cbranch_scc0 .Lskip%=\n\t"
+                         "v_mfma_scale_f32_32x32x64_f8f6f4 %0, %1, %2, %0, %3, %4 op_sel_hi:[0,0,0] cbsz:4 blgp:4\n.Lskip%=:"
+                         : "+a"(acc) : "v"(w), "v"(a), "v"(sw), "v"(sa), "s"(live), "n"(BIT < 0 ? 0 : BIT) : "scc");
+        else
+            asm volatile("s_bitcmp1_b32 %5, %6\n\ts_cbranch_scc0 .Lskip%=\n\t"
+                         "v_mfma_scale_f32_32x32x64_f8f6f4 %0, %1, %2, %0, %3, %4 op_sel_hi:[1,1,0] cbsz:4 blgp:4\n.Lskip%=:"
+                         : "+a"(acc) : "v"(w), "v"(a), "v"(sw), "v"(sa), "s"(live), "n"(BIT < 0 ? 0 : BIT) : "scc");
+    }
+}
+
+// WW x WM = 2 x 2 (dense) or 4 x 1 (grouped: skips the MFMAs of activation blocks without valid rows)
+template <int EPI, int WW, int WM>
+__global__ __launch_bounds__(256) void mx_gemm_pipe_fp4_kernel(const GemmParams p) {
+    static_assert((WW == 2 && WM == 2) || (WW == 4 && WM == 1), "wavefront layout");
+    constexpr int TW = 256, TM = 256, NW = 4, FW = TW / WW / 32, FM = TM / WM / 32, NF = FW + FM;
+    constexpr int kM = FW * FM;                                // 16 MFMAs per step and wavefront
+    constexpr bool kMOuter = FM > FW;
+    constexpr bool kSkip = WM == 1;
+    constexpr int kRows = TW + TM;
+    constexpr int kSlotBytes = kRows * kSlabBytes;            // 64 KiB
+    constexpr int kScaleBase = 2 * kSlotBytes;
+    constexpr int kScaleSlotBytes = kRows * 16;               // one block: 16 bytes (the scales of two slabs) per row
+    constexpr int kTileLoads = kRows / (8 * NW);              // 16
+    constexpr int kWTileLoads = TW / (8 * NW);
+    static_assert(kM == 16 && NF + NF / 2 < kM, "schedule is written for 16 MFMAs per step");
+
+    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+    const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t*)smem;
+
+    const uint32_t tid = threadIdx.x;
+    const uint32_t lane = tid & 63u;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const uint32_t ww = wave % WW, wm = wave / WW;
+    const uint32_t l32 = lane & 31u, lh = lane >> 5;
+
+    Tile tc;
+    if (!locate_tile<TM>(p, tc)) return;
+    const uint32_t g = __builtin_amdgcn_readfirstlane(tc.g), wt = __builtin_amdgcn_readfirstlane(tc.wt);
+    const uint32_t row0 = __builtin_amdgcn_readfirstlane(tc.row0);
+    const uint32_t rows_valid = __builtin_amdgcn_readfirstlane(tc.rows_valid);
+
+    // global row of tile row r (rows past the edge re-read the last valid row; their results are never stored)
+    auto wrow_of = [&](uint32_t r) -> uint32_t {
+        uint32_t gr;
+        if (epi_pairs_gate_up(EPI)) {
+            const uint32_t half = p.n >> 1;
+            uint32_t rr = r < TW / 2 ? wt * (TW / 2) + r : wt * (TW / 2) + (r - TW / 2);
+            rr = rr < half ? rr : half - 1;
+            gr = r < TW / 2 ? rr : half + rr;
+        } else {
+            gr = wt * TW + r;
+            gr = gr < p.n ? gr : p.n - 1;
+        }
+        return gr;
+    };
+    auto arow_of = [&](uint32_t r) -> uint32_t { return r < rows_valid ? r : rows_valid - 1; };
+
+    // LDS-DMA load i of this wavefront fills combined tile rows (4i + wave)*8 .. +8; lane q -> row +q/8, LDS chunk
+    // q%8, and fetches the global chunk that the XOR swizzle maps there
+    uint32_t goff[kTileLoads];
+#pragma unroll
+    for (int i = 0; i < kTileLoads; ++i) {
+        const uint32_t cr = (NW * i + wave) * 8 + (lane >> 3);
+        const uint32_t logical = swz(cr, lane & 7u);
+        goff[i] = (i < kWTileLoads ? mul_lo_u32(wrow_of(cr), p.ldw) : mul_lo_u32(arow_of(cr - TW), p.lda)) + logical * 16;
+    }
+    const uint32_t sgoff_w = wrow_of(64 * wave + lane) * p.ld_ws;
+    const uint32_t sgoff_a = arow_of(64 * wave + lane) * p.ld_as;
+
+    auto make_rsrc = [](const uint8_t* q) -> v4i {
+        const uint64_t v = reinterpret_cast<uint64_t>(q);
+        v4i r;
+        r[0] = __builtin_amdgcn_readfirstlane((int)(uint32_t)v);
+        r[1] = __builtin_amdgcn_readfirstlane((int)(uint32_t)(v >> 32));     // stride 0
+        r[2] = -1;                                                           // no range limit
+        r[3] = 0x00020000;
+        return r;
+    };
+    const v4i w_rs = make_rsrc(p.w + (size_t)g * p.n * p.ldw), a_rs = make_rsrc(p.a + (size_t)row0 * p.lda);
+    const v4i ws_rs = make_rsrc(p.w_scale + (size_t)g * p.n * p.ld_ws), as_rs = make_rsrc(p.a_scale + (size_t)row0 * p.ld_as);
+
+    const uint32_t nslab = p.kbytes / kSlabBytes;
+    const uint32_t dma_base = __builtin_amdgcn_readfirstlane(lds0 + wave * 1024);
+    const uint32_t sdma_base = __builtin_amdgcn_readfirstlane(lds0 + kScaleBase + wave * 64 * 16);
+    const uint32_t sdma_base_a = __builtin_amdgcn_readfirstlane(lds0 + kScaleBase + (TW + wave * 64) * 16);
+
+    auto issue_tile_load = [&](int slot, int i, uint32_t slab) {
+        dma_b128(dma_base + slot * kSlotBytes + i * (NW * 1024), goff[i], i < kWTileLoads ? w_rs : a_rs, slab * kSlabBytes);
+    };
+    // block `blk` (the scales of slabs 2 blk and 2 blk + 1) into ring position blk & 1
+    const uint32_t nblk = nslab / 2;
+    auto issue_scale_block = [&](uint32_t blk) {
+        dma_b128(sdma_base + (blk & 1u) * kScaleSlotBytes, sgoff_w, ws_rs, blk * 16);
+        dma_b128(sdma_base_a + (blk & 1u) * kScaleSlotBytes, sgoff_a, as_rs, blk * 16);
+    };
+    auto clamp_slab = [&](uint32_t slab) -> uint32_t { return slab < nslab ? slab : nslab - 1; };   // past the end: harmless reload
+
+    // fragment read addresses: step h reads the 16-byte chunk 2h + lh of the lane's row
+    const uint32_t x = (l32 & 7u) ^ ((l32 >> 3) & 1u);
+    const uint32_t w_row_base = epi_pairs_gate_up(EPI) ? ww * (TW / 2 / WW) : ww * (TW / WW);
+    uint32_t wb[2][4], ab[2][4];       // [slot][step]
+#pragma unroll
+    for (int s = 0; s < 2; ++s)
+#pragma unroll
+        for (int h = 0; h < 4; ++h) {
+            const uint32_t ch = ((2 * h + lh) ^ x) * 16;
+            wb[s][h] = lds0 + s * kSlotBytes + (w_row_base + l32) * kSlabBytes + ch;
+            ab[s][h] = lds0 + s * kSlotBytes + (TW + wm * (TM / WM) + l32) * kSlabBytes + ch;
+        }
+    const uint32_t swb = lds0 + kScaleBase + (w_row_base + l32) * 16;
+    const uint32_t sab = lds0 + kScaleBase + (TW + wm * (TM / WM) + l32) * 16;
+    const uint32_t sshift = 8 * lh;
+
+    v16f acc[FW][FM];
+#pragma unroll
+    for (int i = 0; i < FW; ++i)
+#pragma unroll
+        for (int j = 0; j < FM; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+
+    v4i fa[NF], fb[NF];                 // the two fragment sets: 0..FW-1 weights, FW.. activations
+    uint32_t sraw[2][NF], scur[2][2][NF];      // [ring slot][dword of the slab][fragment]
+
+#define CMX_PIPE_WOFF(f) ((epi_pairs_gate_up(EPI) ? ((f) < FW / 2 ? (f) * 32 : TW / 2 + ((f) - FW / 2) * 32) : (f) * 32))
+    auto read_piece = [&](auto slot_c, auto step_c, auto pos_c, v4i (&f)[NF]) {
+        constexpr int slot = decltype(slot_c)::value, step = decltype(step_c)::value;
+        constexpr int idx = pipe_read_order<FW, FM>(decltype(pos_c)::value);
+        (void)wb, (void)ab;
+        if constexpr (idx < FW) f[idx] = lds_read_b128<CMX_PIPE_WOFF(idx) * kSlabBytes>(wb[slot][step]);
+        else f[idx] = lds_read_b128<(idx - FW) * 32 * kSlabBytes>(ab[slot][step]);
+    };
+    // dword d of the slab whose scales sit at swb_at / sab_at (= base + ring position + 8 * (slab & 1))
+    auto read_scale = [&](uint32_t swb_at, uint32_t sab_at, auto d_c, auto idx_c) {
+        constexpr int d = decltype(d_c)::value, idx = decltype(idx_c)::value;
+        (void)sraw;
+        if constexpr (idx < FW)
+            sraw[d][idx] = lds_read_b32<CMX_PIPE_WOFF(idx) * 16 + d * 4>(swb_at);
+        else
+            sraw[d][idx] = lds_read_b32<(idx - FW) * 32 * 16 + d * 4>(sab_at);
+    };
+    auto scale_offset_of = [&](uint32_t slab) -> uint32_t {
+        return __builtin_amdgcn_readfirstlane(((slab >> 1) & 1u) * kScaleSlotBytes + (slab & 1u) * 8);
+    };
+    auto shift_scales = [&](auto set_c) {
+        constexpr int set = decltype(set_c)::value;
+        (void)scur, (void)sraw, (void)sshift;
+#pragma unroll
+        for (int d = 0; d < 2; ++d)
+#pragma unroll
+            for (int i = 0; i < NF; ++i)
+                asm volatile("v_lshrrev_b32 %0, %1, %2" : "=v"(scur[set][d][i]) : "v"(sshift), "v"(sraw[d][i]));
+        asm volatile("s_nop 1" ::: "memory");
+    };
+    auto pin_fragments = [&](v4i (&f)[NF]) {
+#pragma unroll
+        for (int i = 0; i < NF; ++i) asm volatile("" ::"v"(f[i]));
+    };
+    auto pin_scales = [&](auto set_c) {
+        constexpr int set = decltype(set_c)::value;
+        (void)scur;
+#pragma unroll
+        for (int d = 0; d < 2; ++d)
+#pragma unroll
+            for (int i = 0; i < NF; ++i) asm volatile("" ::"v"(scur[set][d][i]));
+    };
+
+    using I0 = std::integral_constant<int, 0>;
+    using I1 = std::integral_constant<int, 1>;
+    using I2 = std::integral_constant<int, 2>;
+    using I3 = std::integral_constant<int, 3>;
+
+    // ---- prologue ------------------------------------------------------------------------------------------
+    // scale blocks first, so that the wait below can leave exactly the tile loads of slab 1 in flight
+    issue_scale_block(0);
+    if (nblk > 1) issue_scale_block(1);
+#pragma unroll
+    for (int i = 0; i < kTileLoads; ++i) issue_tile_load(0, i, 0);
+    {
+        const uint32_t k1 = clamp_slab(1);
+#pragma unroll
+        for (int i = 0; i < kTileLoads; ++i) issue_tile_load(1, i, k1);
+    }
+    asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(kTileLoads) : "memory");      // slab 0 and its scales have landed everywhere
+    static_for<0, NF>([&](auto ic) { read_piece(I0{}, I0{}, ic, fa); });
+    static_for<0, NF>([&](auto ic) {
+        read_scale(swb, sab, I0{}, ic);
+        read_scale(swb, sab, I1{}, ic);
+    });
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    shift_scales(I0{});
+
+    const uint32_t live = __builtin_amdgcn_readfirstlane((1u << ((rows_valid + 31) / 32)) - 1u);   // bit fm: block has valid rows
+    // step h of the slab in ring slot `set`: scale dword h/2, byte pair 2*(h%2)
+    auto step_mfma = [&](auto h_c, auto i_c, v4i (&f)[NF], auto set_c) {
+        constexpr int h = decltype(h_c)::value, i = decltype(i_c)::value, set = decltype(set_c)::value;
+        constexpr int fw = kMOuter ? i % FW : i / FM, fm = kMOuter ? i / FW : i % FM;
+        (void)scur, (void)acc;
+        mfma_acc_fp4<(h & 1) * 2, kSkip ? fm : -1>(acc[fw][fm], f[fw], f[FW + fm], scur[set][h >> 1][fw], scur[set][h >> 1][FW + fm], live);
+    };
+
+    constexpr int kB1 = 9;                      // MFMA of step 2 after which the reads of step 3 have landed
+    constexpr int kEarly = kM - kB1 - 1;        // tile loads of slab s+2 issued in step 2 (6)
+    auto slab_body = [&](auto slot_c, uint32_t s) {
+        constexpr int slot = decltype(slot_c)::value;
+        using SlotT = std::integral_constant<int, slot>;
+        using OtherT = std::integral_constant<int, slot ^ 1>;
+        const uint32_t q2 = clamp_slab(s + 2);
+        const uint32_t sc_off = scale_offset_of(s + 1);          // where the scales of the next slab sit
+        const uint32_t swb_at = swb + sc_off, sab_at = sab + sc_off;
+        // ---- steps 0 and 1 ----
+        static_for<0, kM>([&](auto ic) {
+            step_mfma(I0{}, ic, fa, SlotT{});
+            if constexpr (decltype(ic)::value < NF) read_piece(SlotT{}, I1{}, ic, fb);
+        });
+        pin_fragments(fa);
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        static_for<0, kM>([&](auto ic) {
+            step_mfma(I1{}, ic, fb, SlotT{});
+            if constexpr (decltype(ic)::value < NF) read_piece(SlotT{}, I2{}, ic, fa);
+        });
+        pin_fragments(fb);
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        // ---- step 2: last reads of the slot, first loads of slab s+2 ----
+        static_for<0, kM>([&](auto ic) {
+            constexpr int i = decltype(ic)::value;
+            step_mfma(I2{}, ic, fa, SlotT{});
+            if constexpr (i < NF) read_piece(SlotT{}, I3{}, ic, fb);
+            if constexpr (i == kB1) asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+            if constexpr (i > kB1) issue_tile_load(slot, i - kB1 - 1, q2);
+        });
+        pin_fragments(fa);
+        // own loads of slab s+1 are complete (only the kEarly loads just issued may be in flight); after the
+        // barrier so are everyone's
+        asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(kEarly) : "memory");
+        // ---- step 3 ----
+        static_for<0, kM>([&](auto ic) {
+            constexpr int i = decltype(ic)::value;
+            step_mfma(I3{}, ic, fb, SlotT{});
+            if constexpr (i + kEarly < kTileLoads) issue_tile_load(slot, i + kEarly, q2);
+            if constexpr (i + kEarly == kTileLoads) {
+                // the load stream is at slab s + 2: block (s + 3) / 2 goes out with every odd one of its slabs (the ring
+                // position it takes was last read one slab earlier)
+                if (((s + 2) & 1u) && (s + 3) / 2 < nblk) issue_scale_block((s + 3) / 2);
+            }
+            if constexpr (i < NF) read_piece(OtherT{}, I0{}, ic, fa);
+            if constexpr (i >= NF && i < NF + NF / 2) {     // 2 NF scale dwords, four per MFMA
+                constexpr int b = (i - NF) * 2;
+                read_scale(swb_at, sab_at, I0{}, std::integral_constant<int, b>{});
+                read_scale(swb_at, sab_at, I1{}, std::integral_constant<int, b>{});
+                read_scale(swb_at, sab_at, I0{}, std::integral_constant<int, b + 1>{});
+                read_scale(swb_at, sab_at, I1{}, std::integral_constant<int, b + 1>{});
+            }
+            if constexpr (i == (NF + NF / 2 + 1 < kM ? NF + NF / 2 + 1 : kM - 1)) {
+                asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+                shift_scales(OtherT{});
+            }
+        });
+        pin_fragments(fb);
+        pin_scales(SlotT{});
+    };
+
+    // The compiler does not see the MFMAs inside the asm statements: every accumulator passes through an asm
+    // statement that holds the wait states between them and the compiler's own accumulator accesses.
+    auto fence_accumulators = [&]() {
+        v16f* const a = &acc[0][0];
+        asm volatile("s_nop 15\n\ts_nop 15" : "+a"(a[0]), "+a"(a[1]), "+a"(a[2]), "+a"(a[3]), "+a"(a[4]), "+a"(a[5]), "+a"(a[6]), "+a"(a[7]));
+        asm volatile("s_nop 15\n\ts_nop 15" : "+a"(a[8]), "+a"(a[9]), "+a"(a[10]), "+a"(a[11]), "+a"(a[12]), "+a"(a[13]), "+a"(a[14]), "+a"(a[15]));
+    };
+    fence_accumulators();
+    for (uint32_t s = 0; s < nslab; s += 2) {      // the host only selects this kernel for an even slab count
+        slab_body(I0{}, s);
+        slab_body(I1{}, s + 1);
+    }
+    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+    fence_accumulators();
+#undef CMX_PIPE_WOFF
+    epilogue<TW, TM, WW, WM, EPI, FW, FM>(p, tc, acc, ww, wm, lane);
+}

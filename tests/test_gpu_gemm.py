@@ -72,14 +72,17 @@ def test_one_hot_rows_copy_weight_rows_exactly():
     assert np.array_equal(c, want)
 
 
-@pytest.mark.parametrize("tw,tm,waves", [(256, 256, 4), (256, 256, 8), (256, 128, 4)])
-@pytest.mark.parametrize("m,n,k", [(256, 256, 256), (130, 300, 640), (64, 512, 7168)])
+@pytest.mark.parametrize("tw,tm,waves", [(256, 256, 4), (256, 256, 5), (256, 256, 8), (256, 128, 4)])
+@pytest.mark.parametrize("m,n,k", [(256, 256, 256), (130, 300, 640), (64, 512, 7168), (256, 256, 512), (300, 520, 1536)])
 def test_dense_fp4_vs_oracle(tw, tm, waves, m, n, k):
     from catccos_amd import _lib
     _lib.load().cmx_debug_force_tile(tw, tm, waves)
     rng = np.random.default_rng(m + n + k)
     aq, asc = O.mx_quant(rng.uniform(-2, 2, (m, k)).astype(np.float32), "E2M1")
     bq, bsc = O.mx_quant(rng.uniform(-2, 2, (n, k)).astype(np.float32), "E2M1")
+    # uniform data gives every block the same scale: spread them so that a misplaced scale byte shows
+    asc = (asc.astype(np.int32) + rng.integers(-3, 4, asc.shape)).astype(np.uint8)
+    bsc = (bsc.astype(np.int32) + rng.integers(-3, 4, bsc.shape)).astype(np.uint8)
     c = _run(aq, asc, bq, bsc, k, "E2M1")
     gold = O.mx_gemm_f32(aq, asc, bq, bsc, "E2M1", "E2M1")
     bad, worst = close_bf16(host(c), gold)

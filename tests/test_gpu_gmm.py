@@ -128,15 +128,21 @@ def test_swiglu_requant_with_groups_about_one_tile_long():
     assert np.array_equal(host(scales), ws2) and np.array_equal(host(codes), wq2)
 
 
-def test_gmm_fp4_ragged_groups():
-    from catccos_amd import ops
+@pytest.mark.parametrize("tile", [None, (256, 256, 4), (256, 256, 5), (256, 256, 8)])
+@pytest.mark.parametrize("k", [512, 1536, 640])
+def test_gmm_fp4_ragged_groups(tile, k):
+    from catccos_amd import ops, _lib
+    if tile:
+        _lib.load().cmx_debug_force_tile(*tile)
     rng = np.random.default_rng(3)
     counts = [40, 0, 129, 300]
-    n, k = 256, 512
+    n = 256
     m = sum(counts)
     aq, asc = O.mx_quant(rng.uniform(-2, 2, (m, k)).astype(np.float32), "E2M1")
+    asc = (asc.astype(np.int32) + rng.integers(-2, 3, asc.shape)).astype(np.uint8)      # no two neighbouring blocks alike
     ws_ = [O.mx_quant(rng.uniform(-2, 2, (n, k)).astype(np.float32), "E2M1") for _ in counts]
     wq, ws = np.stack([q for q, _ in ws_]), np.stack([s for _, s in ws_])
+    ws = (ws.astype(np.int32) + rng.integers(-2, 3, ws.shape)).astype(np.uint8)
     c = ops.mx_gmm(dev(O.pack_fp4(aq)), dev(asc), dev(O.pack_fp4(wq)), dev(ws), dev(np.array(counts, dtype=np.int32)), k,
                    "E2M1", "fp16")
     gold = O.mx_gmm_f32(aq, asc, wq, ws, counts, "E2M1", "E2M1")
