@@ -996,13 +996,21 @@ int launch_gemm_pipe(const GemmParams& p, uint32_t max_m_tiles, hipStream_t s) {
 
 template <int EPI, int WW, int WM>
 int launch_gemm_pipe_fp4(const GemmParams& p, uint32_t max_m_tiles, hipStream_t s) {
-    constexpr size_t smem = 2 * 512 * kSlabBytes + 2 * 512 * 16;     // tile ring, ring of two scale blocks
+    constexpr size_t smem = 2 * 512 * kSlabBytes + 2 * 512 * 16 + 16;     // tile ring, ring of two scale blocks, next-tile mailbox
     auto kfn = mx_gemm_pipe_fp4_kernel<EPI, WW, WM>;
     static PerDeviceFlag lds_allowed;
     if (int rc = allow_dynamic_lds(kfn, smem, lds_allowed); rc != CMX_OK) return rc;
     const uint64_t tiles = (uint64_t)max_m_tiles * p.w_tiles;
     CMX_REQUIRE(tiles > 0 && tiles < (1ull << 31), "tile count out of range");
-    hipLaunchKernelGGL(kfn, dim3((uint32_t)tiles), dim3(256), smem, s, p);
+    uint32_t grid = (uint32_t)tiles;
+    if (pipe_is_persistent(2, EPI)) {
+        // persistent: one workgroup per CU (the LDS footprint admits no second one), a multiple of the XCD count
+        int cus = 0;
+        if (int rc = cu_count(&cus); rc != CMX_OK) return rc;
+        grid = (uint32_t)(cus / kXcds * kXcds);
+        if (grid < (uint32_t)kXcds) grid = kXcds;
+    }
+    hipLaunchKernelGGL(kfn, dim3(grid), dim3(256), smem, s, p);
     CMX_LAUNCH_CHECK();
     return CMX_OK;
 }
@@ -1067,8 +1075,14 @@ int launch_tile(const GemmParams& p, int waves, uint32_t max_m_tiles, hipStream_
     if constexpr (TW == 256 && TM == 256 && FMT == CMX_FMT_E2M1) {
         // hand-scheduled FP4 kernel: whole two-slab scale blocks (K a multiple of 512 elements), 16-byte aligned scale rows
         if ((waves == 4 || waves == 5) && stream_ok && p.scale_vec16 && p.kbytes % (2 * kSlabBytes) == 0) {
-            if (waves == 4) return launch_gemm_pipe_fp4<EPI, 2, 2>(p, max_m_tiles, s);
-            return launch_gemm_pipe_fp4<EPI, 4, 1>(p, max_m_tiles, s);
+            if constexpr (EPI == kEpiStore) {
+                // plain bf16 output with 4-element-aligned rows: lean store epilogue, persistent kernel
+                const bool lean = p.out_type == CMX_OUT_BF16 && p.n % 4 == 0 && p.ldc % 4 == 0 && (reinterpret_cast<uintptr_t>(p.c) & 7u) == 0;
+                // (as with the 8-bit kernel the 4 x 1 layout would spill inside the loop: the persistent kernel is 2 x 2)
+                if (lean) return launch_gemm_pipe_fp4<kEpiStoreBf16, 2, 2>(p, max_m_tiles, s);
+                if (waves == 4) return launch_gemm_pipe_fp4<EPI, 2, 2>(p, max_m_tiles, s);
+                return launch_gemm_pipe_fp4<EPI, 4, 1>(p, max_m_tiles, s);
+            }
         }
     }
     if constexpr (TW == 256 && TM == 128 && FMT != CMX_FMT_E2M1) {

@@ -13,6 +13,9 @@
 //              the wait for the own loads of slab s+1 and the barrier that publishes it;
 //   step 3:    the other 10 tile loads of slab s+2 (and, every second slab, the next scale block), the reads of
 //              step 0 of slab s+1 from the other slot, its 16 scale dwords and their per-half-wave byte shift.
+// With the lean bf16 store epilogue the kernel is persistent like its 8-bit counterpart: one workgroup per CU walks
+// the tiles of its XCD's run and carries the load stream across tile boundaries, so that the first slabs of a tile
+// arrive while the previous tile's epilogue runs.  With the general store epilogue it takes one tile per workgroup.
 #pragma once
 
 template <int SEL, int BIT>
@@ -42,6 +45,7 @@ __device__ __forceinline__ void mfma_acc_fp4(v16f& acc, const v4i& w, const v4i&
 template <int EPI, int WW, int WM>
 __global__ __launch_bounds__(256) void mx_gemm_pipe_fp4_kernel(const GemmParams p) {
     static_assert((WW == 2 && WM == 2) || (WW == 4 && WM == 1), "wavefront layout");
+    static_assert(!epi_pairs_gate_up(EPI), "store epilogues only");
     constexpr int TW = 256, TM = 256, NW = 4, FW = TW / WW / 32, FM = TM / WM / 32, NF = FW + FM;
     constexpr int kM = FW * FM;                                // 16 MFMAs per step and wavefront
     constexpr bool kMOuter = FM > FW;
@@ -63,40 +67,21 @@ __global__ __launch_bounds__(256) void mx_gemm_pipe_fp4_kernel(const GemmParams 
     const uint32_t ww = wave % WW, wm = wave / WW;
     const uint32_t l32 = lane & 31u, lh = lane >> 5;
 
-    Tile tc;
-    if (!locate_tile<TM>(p, tc)) return;
-    const uint32_t g = __builtin_amdgcn_readfirstlane(tc.g), wt = __builtin_amdgcn_readfirstlane(tc.wt);
-    const uint32_t row0 = __builtin_amdgcn_readfirstlane(tc.row0);
-    const uint32_t rows_valid = __builtin_amdgcn_readfirstlane(tc.rows_valid);
+    // ---- tile sequence of this workgroup (see mx_gemm_pipe_kernel) ----
+    constexpr bool kPersistent = pipe_is_persistent(2, EPI);
+    const uint32_t m_tiles_all = count_m_tiles<TM>(p);
+    const uint32_t total_tiles = m_tiles_all * p.w_tiles;
+    uint32_t run_count;
+    const uint32_t run_first = xcd_run(total_tiles, blockIdx.x % kXcds, run_count);
+    const uint32_t run_end = run_first + run_count;
+    const uint32_t tile_stride = kPersistent ? gridDim.x / kXcds : total_tiles;
+    uint32_t tile_id = run_first + blockIdx.x / kXcds;
+    if (tile_id >= run_end) return;
 
-    // global row of tile row r (rows past the edge re-read the last valid row; their results are never stored)
-    auto wrow_of = [&](uint32_t r) -> uint32_t {
-        uint32_t gr;
-        if (epi_pairs_gate_up(EPI)) {
-            const uint32_t half = p.n >> 1;
-            uint32_t rr = r < TW / 2 ? wt * (TW / 2) + r : wt * (TW / 2) + (r - TW / 2);
-            rr = rr < half ? rr : half - 1;
-            gr = r < TW / 2 ? rr : half + rr;
-        } else {
-            gr = wt * TW + r;
-            gr = gr < p.n ? gr : p.n - 1;
-        }
-        return gr;
-    };
-    auto arow_of = [&](uint32_t r) -> uint32_t { return r < rows_valid ? r : rows_valid - 1; };
-
-    // LDS-DMA load i of this wavefront fills combined tile rows (4i + wave)*8 .. +8; lane q -> row +q/8, LDS chunk
-    // q%8, and fetches the global chunk that the XOR swizzle maps there
-    uint32_t goff[kTileLoads];
-#pragma unroll
-    for (int i = 0; i < kTileLoads; ++i) {
-        const uint32_t cr = (NW * i + wave) * 8 + (lane >> 3);
-        const uint32_t logical = swz(cr, lane & 7u);
-        goff[i] = (i < kWTileLoads ? mul_lo_u32(wrow_of(cr), p.ldw) : mul_lo_u32(arow_of(cr - TW), p.lda)) + logical * 16;
-    }
-    const uint32_t sgoff_w = wrow_of(64 * wave + lane) * p.ld_ws;
-    const uint32_t sgoff_a = arow_of(64 * wave + lane) * p.ld_as;
-
+    // addressing of the tile whose slabs are being requested (switches two slabs before a tile boundary)
+    Tile tq;
+    v4i w_rs, a_rs, ws_rs, as_rs;
+    uint32_t goff[kTileLoads], sgoff_w, sgoff_a;
     auto make_rsrc = [](const uint8_t* q) -> v4i {
         const uint64_t v = reinterpret_cast<uint64_t>(q);
         v4i r;
@@ -106,8 +91,36 @@ __global__ __launch_bounds__(256) void mx_gemm_pipe_fp4_kernel(const GemmParams 
         r[3] = 0x00020000;
         return r;
     };
-    const v4i w_rs = make_rsrc(p.w + (size_t)g * p.n * p.ldw), a_rs = make_rsrc(p.a + (size_t)row0 * p.lda);
-    const v4i ws_rs = make_rsrc(p.w_scale + (size_t)g * p.n * p.ld_ws), as_rs = make_rsrc(p.a_scale + (size_t)row0 * p.ld_as);
+    auto aim_loads_at = [&](uint32_t L) {
+        decode_tile<TM>(p, m_tiles_all, L, tq);
+        const uint32_t g = __builtin_amdgcn_readfirstlane(tq.g), wt = __builtin_amdgcn_readfirstlane(tq.wt);
+        const uint32_t row0 = __builtin_amdgcn_readfirstlane(tq.row0);
+        const uint32_t rows_valid = __builtin_amdgcn_readfirstlane(tq.rows_valid);
+        tq.g = g; tq.wt = wt; tq.row0 = row0; tq.rows_valid = rows_valid;
+        tq.mt = __builtin_amdgcn_readfirstlane(tq.mt);
+        w_rs = make_rsrc(p.w + (size_t)g * p.n * p.ldw);
+        ws_rs = make_rsrc(p.w_scale + (size_t)g * p.n * p.ld_ws);
+        a_rs = make_rsrc(p.a + (size_t)row0 * p.lda);
+        as_rs = make_rsrc(p.a_scale + (size_t)row0 * p.ld_as);
+        // global row of tile row r (rows past the edge re-read the last valid row; their results are never stored)
+        auto wrow_of = [&](uint32_t r) -> uint32_t {
+            const uint32_t gr = wt * TW + r;
+            return gr < p.n ? gr : p.n - 1;
+        };
+        auto arow_of = [&](uint32_t r) -> uint32_t { return r < rows_valid ? r : rows_valid - 1; };
+        // LDS-DMA load i of this wavefront fills combined tile rows (4i + wave)*8 .. +8; lane q -> row +q/8, LDS
+        // chunk q%8, and fetches the global chunk that the XOR swizzle maps there
+#pragma unroll
+        for (int i = 0; i < kTileLoads; ++i) {
+            const uint32_t cr = (NW * i + wave) * 8 + (lane >> 3);
+            const uint32_t logical = swz(cr, lane & 7u);
+            goff[i] = (i < kWTileLoads ? mul_lo_u32(wrow_of(cr), p.ldw) : mul_lo_u32(arow_of(cr - TW), p.lda)) + logical * 16;
+        }
+        sgoff_w = wrow_of(64 * wave + lane) * p.ld_ws;
+        sgoff_a = arow_of(64 * wave + lane) * p.ld_as;
+    };
+    aim_loads_at(tile_id);
+    Tile tc = tq;                               // tile of the MFMA stream / epilogue
 
     const uint32_t nslab = p.kbytes / kSlabBytes;
     const uint32_t dma_base = __builtin_amdgcn_readfirstlane(lds0 + wave * 1024);
@@ -117,12 +130,19 @@ __global__ __launch_bounds__(256) void mx_gemm_pipe_fp4_kernel(const GemmParams 
     auto issue_tile_load = [&](int slot, int i, uint32_t slab) {
         dma_b128(dma_base + slot * kSlotBytes + i * (NW * 1024), goff[i], i < kWTileLoads ? w_rs : a_rs, slab * kSlabBytes);
     };
-    // block `blk` (the scales of slabs 2 blk and 2 blk + 1) into ring position blk & 1
+    // block `blk` of the load stream's tile (the scales of its slabs 2 blk and 2 blk + 1) into the next ring position
     const uint32_t nblk = nslab / 2;
+    uint32_t blocks_issued = 0;          // running count over all tiles of this workgroup: ring position = count & 1
     auto issue_scale_block = [&](uint32_t blk) {
-        dma_b128(sdma_base + (blk & 1u) * kScaleSlotBytes, sgoff_w, ws_rs, blk * 16);
-        dma_b128(sdma_base_a + (blk & 1u) * kScaleSlotBytes, sgoff_a, as_rs, blk * 16);
+        const uint32_t pos = blocks_issued & 1u;
+        ++blocks_issued;
+        dma_b128(sdma_base + pos * kScaleSlotBytes, sgoff_w, ws_rs, blk * 16);
+        dma_b128(sdma_base_a + pos * kScaleSlotBytes, sgoff_a, as_rs, blk * 16);
     };
+    // the load stream is at slab q of its tile: block 0 goes out with slab 0, block b with slab 2b - 1 (the ring
+    // position it takes was last read one slab earlier)
+    auto scale_block_due = [&](uint32_t q) -> bool { return q == 0 || ((q & 1u) && (q + 1) / 2 < nblk); };
+    auto scale_block_of = [&](uint32_t q) -> uint32_t { return (q + 1) / 2; };
     auto clamp_slab = [&](uint32_t slab) -> uint32_t { return slab < nslab ? slab : nslab - 1; };   // past the end: harmless reload
 
     // fragment read addresses: step h reads the 16-byte chunk 2h + lh of the lane's row
@@ -169,8 +189,11 @@ __global__ __launch_bounds__(256) void mx_gemm_pipe_fp4_kernel(const GemmParams 
         else
             sraw[d][idx] = lds_read_b32<(idx - FW) * 32 * 16 + d * 4>(sab_at);
     };
-    auto scale_offset_of = [&](uint32_t slab) -> uint32_t {
-        return __builtin_amdgcn_readfirstlane(((slab >> 1) & 1u) * kScaleSlotBytes + (slab & 1u) * 8);
+    // running index (over all tiles) of the slab whose scales are read next: its block sits at ring position
+    // (index / 2) & 1, its two dwords at 8 * (index & 1)
+    uint32_t scale_read_slab = 0;
+    auto scale_read_offset = [&]() -> uint32_t {
+        return __builtin_amdgcn_readfirstlane(((scale_read_slab >> 1) & 1u) * kScaleSlotBytes + (scale_read_slab & 1u) * 8);
     };
     auto shift_scales = [&](auto set_c) {
         constexpr int set = decltype(set_c)::value;
@@ -212,15 +235,23 @@ __global__ __launch_bounds__(256) void mx_gemm_pipe_fp4_kernel(const GemmParams 
         for (int i = 0; i < kTileLoads; ++i) issue_tile_load(1, i, k1);
     }
     asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(kTileLoads) : "memory");      // slab 0 and its scales have landed everywhere
-    static_for<0, NF>([&](auto ic) { read_piece(I0{}, I0{}, ic, fa); });
-    static_for<0, NF>([&](auto ic) {
-        read_scale(swb, sab, I0{}, ic);
-        read_scale(swb, sab, I1{}, ic);
-    });
-    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-    shift_scales(I0{});
+    // step 0 of the slab in slot 0 and its scales into fragment set a / scale set 0
+    auto read_first_step = [&]() {
+        static_for<0, NF>([&](auto ic) { read_piece(I0{}, I0{}, ic, fa); });
+        const uint32_t off = scale_read_offset();
+        const uint32_t swb_at = swb + off, sab_at = sab + off;
+        static_for<0, NF>([&](auto ic) {
+            read_scale(swb_at, sab_at, I0{}, ic);
+            read_scale(swb_at, sab_at, I1{}, ic);
+        });
+        ++scale_read_slab;
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        shift_scales(I0{});
+    };
+    read_first_step();
 
-    const uint32_t live = __builtin_amdgcn_readfirstlane((1u << ((rows_valid + 31) / 32)) - 1u);   // bit fm: block has valid rows
+    auto live_mask = [](uint32_t rows_valid) -> uint32_t { return __builtin_amdgcn_readfirstlane((1u << ((rows_valid + 31) / 32)) - 1u); };
+    uint32_t live = live_mask(tc.rows_valid);      // bit fm: activation block fm has valid rows
     // step h of the slab in ring slot `set`: scale dword h/2, byte pair 2*(h%2)
     auto step_mfma = [&](auto h_c, auto i_c, v4i (&f)[NF], auto set_c) {
         constexpr int h = decltype(h_c)::value, i = decltype(i_c)::value, set = decltype(set_c)::value;
@@ -231,13 +262,15 @@ __global__ __launch_bounds__(256) void mx_gemm_pipe_fp4_kernel(const GemmParams 
 
     constexpr int kB1 = 9;                      // MFMA of step 2 after which the reads of step 3 have landed
     constexpr int kEarly = kM - kB1 - 1;        // tile loads of slab s+2 issued in step 2 (6)
-    auto slab_body = [&](auto slot_c, uint32_t s) {
+    constexpr uint32_t kNoSlab = 0xFFFFFFFFu;
+    // q = slab of the load stream within its tile (kNoSlab: nothing new to request, slab q2 is requested again)
+    auto slab_body = [&](auto slot_c, uint32_t q2, uint32_t q) {
         constexpr int slot = decltype(slot_c)::value;
         using SlotT = std::integral_constant<int, slot>;
         using OtherT = std::integral_constant<int, slot ^ 1>;
-        const uint32_t q2 = clamp_slab(s + 2);
-        const uint32_t sc_off = scale_offset_of(s + 1);          // where the scales of the next slab sit
+        const uint32_t sc_off = scale_read_offset();             // where the scales of the next slab sit
         const uint32_t swb_at = swb + sc_off, sab_at = sab + sc_off;
+        ++scale_read_slab;
         // ---- steps 0 and 1 ----
         static_for<0, kM>([&](auto ic) {
             step_mfma(I0{}, ic, fa, SlotT{});
@@ -269,9 +302,7 @@ __global__ __launch_bounds__(256) void mx_gemm_pipe_fp4_kernel(const GemmParams 
             step_mfma(I3{}, ic, fb, SlotT{});
             if constexpr (i + kEarly < kTileLoads) issue_tile_load(slot, i + kEarly, q2);
             if constexpr (i + kEarly == kTileLoads) {
-                // the load stream is at slab s + 2: block (s + 3) / 2 goes out with every odd one of its slabs (the ring
-                // position it takes was last read one slab earlier)
-                if (((s + 2) & 1u) && (s + 3) / 2 < nblk) issue_scale_block((s + 3) / 2);
+                if (q != kNoSlab && scale_block_due(q)) issue_scale_block(scale_block_of(q));
             }
             if constexpr (i < NF) read_piece(OtherT{}, I0{}, ic, fa);
             if constexpr (i >= NF && i < NF + NF / 2) {     // 2 NF scale dwords, four per MFMA
@@ -297,13 +328,67 @@ __global__ __launch_bounds__(256) void mx_gemm_pipe_fp4_kernel(const GemmParams 
         asm volatile("s_nop 15\n\ts_nop 15" : "+a"(a[0]), "+a"(a[1]), "+a"(a[2]), "+a"(a[3]), "+a"(a[4]), "+a"(a[5]), "+a"(a[6]), "+a"(a[7]));
         asm volatile("s_nop 15\n\ts_nop 15" : "+a"(a[8]), "+a"(a[9]), "+a"(a[10]), "+a"(a[11]), "+a"(a[12]), "+a"(a[13]), "+a"(a[14]), "+a"(a[15]));
     };
-    fence_accumulators();
-    for (uint32_t s = 0; s < nslab; s += 2) {      // the host only selects this kernel for an even slab count
-        slab_body(I0{}, s);
-        slab_body(I1{}, s + 1);
+    fence_accumulators();       // the zero initialisation has retired before the first MFMA reads it
+    if constexpr (!kPersistent) {
+        for (uint32_t s = 0; s < nslab; s += 2) {      // the host only selects this kernel for an even slab count
+            const uint32_t q0 = s + 2, q1 = s + 3;
+            slab_body(I0{}, clamp_slab(q0), q0 < nslab ? q0 : kNoSlab);
+            slab_body(I1{}, clamp_slab(q1), q1 < nslab ? q1 : kNoSlab);
+        }
+        asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+        fence_accumulators();
+        epilogue<TW, TM, WW, WM, EPI, FW, FM>(p, tc, acc, ww, wm, lane);
+    } else {
+        // The load stream runs two slabs ahead of the MFMA stream: at the end of a tile it is aimed at the
+        // workgroup's next tile (or keeps requesting the last slab again when there is none).  With a counter
+        // array (grouped problems) the workgroups of an XCD draw their next tile from that XCD's run in order.
+        uint32_t sm = 0;             // slab of the MFMA stream within its tile
+        uint32_t sq = 2;             // slab of the load stream within its tile
+        bool next_ok = false;        // the load stream has moved on to a next tile
+        uint32_t next_id = tile_id;
+        for (;;) {
+            if (sq == nslab) {
+                if (p.tile_ctr != nullptr) {
+                    uint32_t* const mailbox = reinterpret_cast<uint32_t*>(smem + kScaleBase + 2 * kScaleSlotBytes);
+                    if (tid == 0) *mailbox = atomicAdd(reinterpret_cast<unsigned int*>(p.tile_ctr) + blockIdx.x % kXcds, 1u);
+                    __syncthreads();
+                    next_id = run_first + tile_stride + __builtin_amdgcn_readfirstlane(*mailbox);
+                } else {
+                    next_id = tile_id + tile_stride;
+                }
+                next_ok = next_id < run_end;
+                if (next_ok) {
+                    aim_loads_at(next_id);
+                    sq = 0;
+                }
+            }
+            slab_body(I0{}, clamp_slab(sq), sq < nslab ? sq : kNoSlab);
+            slab_body(I1{}, clamp_slab(sq + 1), sq + 1 < nslab ? sq + 1 : kNoSlab);
+            sq += 2;
+            sm += 2;
+            if (sm == nslab) {
+                fence_accumulators();           // the last MFMAs have written their accumulators
+                epilogue<TW, TM, WW, WM, EPI, FW, FM>(p, tc, acc, ww, wm, lane);
+                if (!next_ok) break;
+                tile_id = next_id;
+                tc = tq;
+                live = live_mask(tc.rows_valid);
+                next_ok = false;
+                sm = 0;
+#pragma unroll
+                for (int i = 0; i < FW; ++i)
+#pragma unroll
+                    for (int j = 0; j < FM; ++j)
+#pragma unroll
+                        for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+                fence_accumulators();
+                // the last slab body has read the new tile's first fragments and scales already; they are not
+                // carried through the epilogue but read again (slot 0, landed)
+                --scale_read_slab;
+                read_first_step();
+            }
+        }
+        asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");     // the re-requested slabs land before the LDS is released
     }
-    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
-    fence_accumulators();
 #undef CMX_PIPE_WOFF
-    epilogue<TW, TM, WW, WM, EPI, FW, FM>(p, tc, acc, ww, wm, lane);
 }
