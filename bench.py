@@ -260,7 +260,7 @@ def main() -> int:
         ws5 = ops.gmm_workspace(E5, dev)
         t5 = hip_time(lambda: ops.mx_gmm(a5, a5s, w5, w5s, c5, K5, "E2M1", "bf16", c=c_out, workspace=ws5))
         fl5 = 2.0 * rows5 * K5 * N5
-        extra["mxfp4_gmm_cfg5"] = {"kernel": "mx_gemm_pipe_fp4_kernel<store epilogue, 2x2 wavefronts> (grouped, 256x256 tile)", "bound": "mfma",
+        extra["mxfp4_gmm_cfg5"] = {"kernel": "mx_gemm_pipe_fp4_kernel<bf16 store epilogue, 2x2 wavefronts, persistent> (grouped, 256x256 tile)", "bound": "mfma",
                                    "achieved": fl5 / t5 / 1e12, "peak": MXFP4_PEAK_TFLOPS, "unit": "TFLOP/s",
                                    "frac": fl5 / t5 / 1e12 / MXFP4_PEAK_TFLOPS, "avg_launch_us": t5 * 1e6}
         log(f"[mxfp4 gmm cfg5] {t5*1e6:.1f} us -> {fl5/t5/1e12:.0f} TFLOP/s")

@@ -1041,8 +1041,8 @@ TileChoice g_force_tile = {0, 0, 0};   // test/tuning hook: tw == 0 -> heuristic
 // than two tiles of rows take 4 x 1, where every wavefront shares in whatever rows a ragged tile has
 // (measured: 16 groups of ~2048 rows 891 vs 918 us in favour of 2 x 2, 256 groups of ~256 rows 4.33 vs
 // 4.38 ms in favour of 4 x 1).  FP4 has its own hand-scheduled kernel in the same two layouts (K a multiple of 512
-// elements; 16 groups of ~2048 rows at K = 7168, N = 4096: 2 x 2 635 us, 4 x 1 700 us, the eight-wavefront
-// streaming kernel, which takes every other FP4 problem, 750 us).
+// elements; 16 groups of ~2048 rows at K = 7168, N = 4096: 2 x 2 persistent 565 us, one tile per workgroup 2 x 2
+// 635 us and 4 x 1 700 us, the eight-wavefront streaming kernel, which takes every other FP4 problem, 750 us).
 TileChoice choose_tile(uint32_t m_hint, uint32_t n, int fmt, bool grouped) {
     if (g_force_tile.tw) return g_force_tile;
     // short problems stream their weights once: the three-slot 256 x 128 kernel keeps two slabs in flight

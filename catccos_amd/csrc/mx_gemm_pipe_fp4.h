@@ -18,6 +18,24 @@
 // arrive while the previous tile's epilogue runs.  With the general store epilogue it takes one tile per workgroup.
 #pragma once
 
+// An LDS-DMA load in two statements, so that a scheduled instruction (an MFMA, an LDS read) can stand where the wait
+// state between the write of M0 and the load would otherwise be an s_nop.  Nothing between the two may write M0.
+__device__ __forceinline__ void dma_aim(uint32_t lds_dst) {
+    lds_dst = __builtin_amdgcn_readfirstlane(lds_dst);
+    asm volatile("s_mov_b32 m0, %0" ::"s"(lds_dst) : "memory");
+}
+__device__ __forceinline__ void dma_b128_aimed(uint32_t voff, v4i rsrc, uint32_t soff) {
+    soff = __builtin_amdgcn_readfirstlane(soff);
+    asm volatile("buffer_load_dwordx4 %0, %1, %2 offen lds" ::"v"(voff), "s"(rsrc), "s"(soff) : "memory");
+}
+typedef int v2i __attribute__((ext_vector_type(2)));
+template <int OFF>
+__device__ __forceinline__ v2i lds_read_b64(uint32_t addr) {
+    v2i r;
+    asm volatile("ds_read_b64 %0, %1 offset:%2" : "=v"(r) : "v"(addr), "n"(OFF) : "memory");
+    return r;
+}
+
 template <int SEL, int BIT>
 __device__ __forceinline__ void mfma_acc_fp4(v16f& acc, const v4i& w, const v4i& a, uint32_t sw, uint32_t sa, uint32_t live) {
     static_assert(SEL == 0 || SEL == 2, "scale byte pair");
@@ -130,6 +148,9 @@ __global__ __launch_bounds__(256) void mx_gemm_pipe_fp4_kernel(const GemmParams 
     auto issue_tile_load = [&](int slot, int i, uint32_t slab) {
         dma_b128(dma_base + slot * kSlotBytes + i * (NW * 1024), goff[i], i < kWTileLoads ? w_rs : a_rs, slab * kSlabBytes);
     };
+    // the same in two halves, with an MFMA between them
+    auto aim_tile_load = [&](int slot, int i) { dma_aim(dma_base + slot * kSlotBytes + i * (NW * 1024)); };
+    auto fire_tile_load = [&](int i, uint32_t slab) { dma_b128_aimed(goff[i], i < kWTileLoads ? w_rs : a_rs, slab * kSlabBytes); };
     // block `blk` of the load stream's tile (the scales of its slabs 2 blk and 2 blk + 1) into the next ring position
     const uint32_t nblk = nslab / 2;
     uint32_t blocks_issued = 0;          // running count over all tiles of this workgroup: ring position = count & 1
@@ -170,7 +191,8 @@ __global__ __launch_bounds__(256) void mx_gemm_pipe_fp4_kernel(const GemmParams 
             for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
 
     v4i fa[NF], fb[NF];                 // the two fragment sets: 0..FW-1 weights, FW.. activations
-    uint32_t sraw[2][NF], scur[2][2][NF];      // [ring slot][dword of the slab][fragment]
+    v2i sraw[NF];                       // the two scale dwords of a slab, as read
+    uint32_t scur[2][2][NF];            // shifted: [ring slot][dword of the slab][fragment]
 
 #define CMX_PIPE_WOFF(f) ((epi_pairs_gate_up(EPI) ? ((f) < FW / 2 ? (f) * 32 : TW / 2 + ((f) - FW / 2) * 32) : (f) * 32))
     auto read_piece = [&](auto slot_c, auto step_c, auto pos_c, v4i (&f)[NF]) {
@@ -180,14 +202,14 @@ __global__ __launch_bounds__(256) void mx_gemm_pipe_fp4_kernel(const GemmParams 
         if constexpr (idx < FW) f[idx] = lds_read_b128<CMX_PIPE_WOFF(idx) * kSlabBytes>(wb[slot][step]);
         else f[idx] = lds_read_b128<(idx - FW) * 32 * kSlabBytes>(ab[slot][step]);
     };
-    // dword d of the slab whose scales sit at swb_at / sab_at (= base + ring position + 8 * (slab & 1))
-    auto read_scale = [&](uint32_t swb_at, uint32_t sab_at, auto d_c, auto idx_c) {
-        constexpr int d = decltype(d_c)::value, idx = decltype(idx_c)::value;
+    // both dwords of the slab whose scales sit at swb_at / sab_at (= base + ring position + 8 * (slab & 1))
+    auto read_scale = [&](uint32_t swb_at, uint32_t sab_at, auto idx_c) {
+        constexpr int idx = decltype(idx_c)::value;
         (void)sraw;
         if constexpr (idx < FW)
-            sraw[d][idx] = lds_read_b32<CMX_PIPE_WOFF(idx) * 16 + d * 4>(swb_at);
+            sraw[idx] = lds_read_b64<CMX_PIPE_WOFF(idx) * 16>(swb_at);
         else
-            sraw[d][idx] = lds_read_b32<(idx - FW) * 32 * 16 + d * 4>(sab_at);
+            sraw[idx] = lds_read_b64<(idx - FW) * 32 * 16>(sab_at);
     };
     // running index (over all tiles) of the slab whose scales are read next: its block sits at ring position
     // (index / 2) & 1, its two dwords at 8 * (index & 1)
@@ -195,15 +217,12 @@ __global__ __launch_bounds__(256) void mx_gemm_pipe_fp4_kernel(const GemmParams 
     auto scale_read_offset = [&]() -> uint32_t {
         return __builtin_amdgcn_readfirstlane(((scale_read_slab >> 1) & 1u) * kScaleSlotBytes + (scale_read_slab & 1u) * 8);
     };
-    auto shift_scales = [&](auto set_c) {
-        constexpr int set = decltype(set_c)::value;
+    // per-half-wave byte shift of fragment idx's scales into set `set`
+    auto shift_scale = [&](auto set_c, auto idx_c) {
+        constexpr int set = decltype(set_c)::value, i = decltype(idx_c)::value;
         (void)scur, (void)sraw, (void)sshift;
-#pragma unroll
-        for (int d = 0; d < 2; ++d)
-#pragma unroll
-            for (int i = 0; i < NF; ++i)
-                asm volatile("v_lshrrev_b32 %0, %1, %2" : "=v"(scur[set][d][i]) : "v"(sshift), "v"(sraw[d][i]));
-        asm volatile("s_nop 1" ::: "memory");
+        asm volatile("v_lshrrev_b32 %0, %1, %2" : "=v"(scur[set][0][i]) : "v"(sshift), "v"(sraw[i][0]));
+        asm volatile("v_lshrrev_b32 %0, %1, %2" : "=v"(scur[set][1][i]) : "v"(sshift), "v"(sraw[i][1]));
     };
     auto pin_fragments = [&](v4i (&f)[NF]) {
 #pragma unroll
@@ -240,13 +259,11 @@ __global__ __launch_bounds__(256) void mx_gemm_pipe_fp4_kernel(const GemmParams 
         static_for<0, NF>([&](auto ic) { read_piece(I0{}, I0{}, ic, fa); });
         const uint32_t off = scale_read_offset();
         const uint32_t swb_at = swb + off, sab_at = sab + off;
-        static_for<0, NF>([&](auto ic) {
-            read_scale(swb_at, sab_at, I0{}, ic);
-            read_scale(swb_at, sab_at, I1{}, ic);
-        });
+        static_for<0, NF>([&](auto ic) { read_scale(swb_at, sab_at, ic); });
         ++scale_read_slab;
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-        shift_scales(I0{});
+        static_for<0, NF>([&](auto ic) { shift_scale(I0{}, ic); });
+        asm volatile("s_nop 1" ::: "memory");      // the first MFMA may be the very next instruction
     };
     read_first_step();
 
@@ -271,52 +288,59 @@ __global__ __launch_bounds__(256) void mx_gemm_pipe_fp4_kernel(const GemmParams 
         const uint32_t sc_off = scale_read_offset();             // where the scales of the next slab sit
         const uint32_t swb_at = swb + sc_off, sab_at = sab + sc_off;
         ++scale_read_slab;
-        // ---- steps 0 and 1 ----
+        // ---- step 0: fragments of step 1; behind them the scales of the next slab (they landed long ago) ----
         static_for<0, kM>([&](auto ic) {
+            constexpr int i = decltype(ic)::value;
             step_mfma(I0{}, ic, fa, SlotT{});
-            if constexpr (decltype(ic)::value < NF) read_piece(SlotT{}, I1{}, ic, fb);
+            if constexpr (i < NF) read_piece(SlotT{}, I1{}, ic, fb);
+            if constexpr (i >= NF && 2 * (i - NF) < NF) {
+                read_scale(swb_at, sab_at, std::integral_constant<int, 2 * (i - NF)>{});
+                if constexpr (2 * (i - NF) + 1 < NF) read_scale(swb_at, sab_at, std::integral_constant<int, 2 * (i - NF) + 1>{});
+            }
         });
         pin_fragments(fa);
-        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        asm volatile("s_waitcnt lgkmcnt(%0)" ::"n"(NF) : "memory");        // LDS reads return in order: all but the NF scale reads
+        // ---- step 1: fragments of step 2; then the byte shifts of the next slab's scales ----
         static_for<0, kM>([&](auto ic) {
+            constexpr int i = decltype(ic)::value;
             step_mfma(I1{}, ic, fb, SlotT{});
-            if constexpr (decltype(ic)::value < NF) read_piece(SlotT{}, I2{}, ic, fa);
+            if constexpr (i < NF) read_piece(SlotT{}, I2{}, ic, fa);
+            if constexpr (i == NF) asm volatile("s_waitcnt lgkmcnt(%0)" ::"n"(NF) : "memory");      // the scale reads, not the NF fragment reads behind them
+            if constexpr (i >= NF) {
+                constexpr int per = (NF + (kM - NF) - 1) / (kM - NF);          // fragments per MFMA
+                static_for<0, per>([&](auto jc) {
+                    constexpr int idx = (i - NF) * per + decltype(jc)::value;
+                    if constexpr (idx < NF) shift_scale(OtherT{}, std::integral_constant<int, idx>{});
+                });
+            }
         });
         pin_fragments(fb);
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
         // ---- step 2: last reads of the slot, first loads of slab s+2 ----
         static_for<0, kM>([&](auto ic) {
             constexpr int i = decltype(ic)::value;
+            if constexpr (i > kB1) aim_tile_load(slot, i - kB1 - 1);
             step_mfma(I2{}, ic, fa, SlotT{});
             if constexpr (i < NF) read_piece(SlotT{}, I3{}, ic, fb);
             if constexpr (i == kB1) asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
-            if constexpr (i > kB1) issue_tile_load(slot, i - kB1 - 1, q2);
+            if constexpr (i > kB1) fire_tile_load(i - kB1 - 1, q2);
         });
         pin_fragments(fa);
         // own loads of slab s+1 are complete (only the kEarly loads just issued may be in flight); after the
         // barrier so are everyone's
         asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(kEarly) : "memory");
-        // ---- step 3 ----
+        // ---- step 3: the other loads, the first fragments of the next slab ----
         static_for<0, kM>([&](auto ic) {
             constexpr int i = decltype(ic)::value;
+            if constexpr (i + kEarly < kTileLoads) aim_tile_load(slot, i + kEarly);
             step_mfma(I3{}, ic, fb, SlotT{});
-            if constexpr (i + kEarly < kTileLoads) issue_tile_load(slot, i + kEarly, q2);
+            if constexpr (i < NF) read_piece(OtherT{}, I0{}, ic, fa);
+            if constexpr (i + kEarly < kTileLoads) fire_tile_load(i + kEarly, q2);
             if constexpr (i + kEarly == kTileLoads) {
                 if (q != kNoSlab && scale_block_due(q)) issue_scale_block(scale_block_of(q));
             }
-            if constexpr (i < NF) read_piece(OtherT{}, I0{}, ic, fa);
-            if constexpr (i >= NF && i < NF + NF / 2) {     // 2 NF scale dwords, four per MFMA
-                constexpr int b = (i - NF) * 2;
-                read_scale(swb_at, sab_at, I0{}, std::integral_constant<int, b>{});
-                read_scale(swb_at, sab_at, I1{}, std::integral_constant<int, b>{});
-                read_scale(swb_at, sab_at, I0{}, std::integral_constant<int, b + 1>{});
-                read_scale(swb_at, sab_at, I1{}, std::integral_constant<int, b + 1>{});
-            }
-            if constexpr (i == (NF + NF / 2 + 1 < kM ? NF + NF / 2 + 1 : kM - 1)) {
-                asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-                shift_scales(OtherT{});
-            }
         });
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");      // fragment set a of the next slab
         pin_fragments(fb);
         pin_scales(SlotT{});
     };
