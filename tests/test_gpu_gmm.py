@@ -71,6 +71,55 @@ def test_gmm_many_ragged_groups_every_row(tile):
     assert np.array_equal(host(scales), ws2) and np.array_equal(host(codes), wq2)
 
 
+@pytest.mark.parametrize("fmt,k", [("E4M3", 512), ("E2M1", 512), ("E2M1", 1024)])
+def test_more_tiles_than_workgroups_every_row(fmt, k):
+    """Enough tiles (about 300 of 256 x 256) that the persistent kernels, one workgroup per CU, walk on to a second
+    tile: the load stream crosses the tile boundary, the next tile comes from the per-XCD counters, and every
+    row of every group must still come out right, with the rows past the groups untouched."""
+    from catccos_amd import ops, _lib
+    _lib.load().cmx_debug_force_tile(256, 256, 4)
+    rng = np.random.default_rng(91)
+    counts = [int(c) for c in rng.integers(0, 700, size=36)] + [256, 512, 0, 128, 1, 255]
+    n = 1024
+    m = sum(counts)
+    if fmt == "E2M1":
+        aq, asc = O.mx_quant(rng.uniform(-2, 2, (m + 3, k)).astype(np.float32), "E2M1")
+        qs = [O.mx_quant(rng.uniform(-2, 2, (n, k)).astype(np.float32), "E2M1") for _ in counts]
+        pack = O.pack_fp4
+    else:
+        aq, asc = O.mx_quant(O.bf16_round(rng.standard_normal((m + 3, k)).astype(np.float32)))
+        qs = [O.mx_quant(O.bf16_round(rng.standard_normal((n, k)).astype(np.float32))) for _ in counts]
+        pack = lambda x: x
+    wq, ws = np.stack([q for q, _ in qs]), np.stack([s_ for _, s_ in qs])
+    c = torch.full((m + 3, n), 7.0, dtype=torch.bfloat16, device="cuda")
+    ops.mx_gmm(dev(pack(aq)), dev(asc), dev(pack(wq)), dev(ws), dev(np.array(counts, dtype=np.int32)), k, fmt, "bf16", c=c)
+    got = host(c)
+    bad, worst = close_bf16(got[:m], O.mx_gmm_f32(aq[:m], asc[:m], wq, ws, counts, fmt, fmt))
+    assert bad == 0, (bad, worst)
+    assert np.all(O.bf16_bits_to_f32(got[m:]) == 7.0)
+
+
+@pytest.mark.parametrize("waves", [4, 5])
+def test_swiglu_requant_more_tiles_than_workgroups(waves):
+    """The fused GMM1 epilogue on about 300 tiles: the persistent kernels (2 x 2 and 4 x 1 wavefronts) go through
+    the epilogue and on to a next tile."""
+    from catccos_amd import ops, _lib
+    _lib.load().cmx_debug_force_tile(256, 256, waves)
+    rng = np.random.default_rng(92)
+    counts = [int(c) for c in rng.integers(0, 700, size=36)] + [256, 512, 0, 128, 1, 255]
+    n, k = 1024, 512
+    m = sum(counts)
+    aq, asc = O.mx_quant(O.bf16_round(rng.standard_normal((m, k)).astype(np.float32)))
+    wq, ws = _weights(rng, len(counts), n, k, std=0.06)
+    codes, scales, act = ops.mx_gmm_swiglu_quant(dev(aq), dev(asc), dev(wq), dev(ws), dev(np.array(counts, dtype=np.int32)), k,
+                                                 want_bf16=True)
+    _, act_g, _, _ = O.gmm1_swiglu_quant(aq, asc, wq, ws, counts)
+    bad, worst = close_bf16(host(act), O.bf16_bits_to_f32(act_g), rtol=2e-2)
+    assert bad == 0, (bad, worst)
+    wq2, ws2 = O.mx_quant_bf16(host(act), "E4M3", "rne")
+    assert np.array_equal(host(scales), ws2) and np.array_equal(host(codes), wq2)
+
+
 @pytest.mark.parametrize("tile", [None, (256, 128, 5), (128, 128, 4)])
 def test_group_sizes_that_overrun_the_buffers_are_cut_off(tile):
     """The sizes are device data the host cannot check: rows past m_total are dropped group by group and negative
