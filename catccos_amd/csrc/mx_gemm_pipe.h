@@ -150,7 +150,7 @@ __global__ __launch_bounds__(256) void mx_gemm_pipe_kernel(const GemmParams p) {
     const uint32_t l32 = lane & 31u, lh = lane >> 5;
 
     // ---- tile sequence of this workgroup ------------------------------------------------------------------
-    // The two-slot kernels with the SwiGLU or the lean bf16 store epilogue are persistent: the grid is one
+    // The two-slot kernels with the SwiGLU or the lean 16-bit store epilogue are persistent: the grid is one
     // workgroup per CU, and workgroup j of XCD x walks tiles j, j + (workgroups per XCD), ... of that XCD's
     // contiguous run, carrying the load pipeline across tile boundaries.  The others take one tile per
     // workgroup (the general store epilogue with its three output types and edge cases needs too many

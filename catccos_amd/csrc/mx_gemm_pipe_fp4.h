@@ -13,7 +13,7 @@
 //              the wait for the own loads of slab s+1 and the barrier that publishes it;
 //   step 3:    the other 10 tile loads of slab s+2 (and, every second slab, the next scale block), the reads of
 //              step 0 of slab s+1 from the other slot, its 16 scale dwords and their per-half-wave byte shift.
-// With the lean bf16 store epilogue the kernel is persistent like its 8-bit counterpart: one workgroup per CU walks
+// With the lean 16-bit store epilogue the kernel is persistent like its 8-bit counterpart: one workgroup per CU walks
 // the tiles of its XCD's run and carries the load stream across tile boundaries, so that the first slabs of a tile
 // arrive while the previous tile's epilogue runs.  With the general store epilogue it takes one tile per workgroup.
 #pragma once
