@@ -143,11 +143,22 @@ __device__ __forceinline__ uint32_t xcd_run(uint32_t total_tiles, uint32_t x, ui
     return x * base + (x < rem ? x : rem);
 }
 
+// g_from: a group at or before the tile's (0, or the group of an earlier tile of an increasing sequence)
 template <int TM>
-__device__ __forceinline__ void decode_tile(const GemmParams& p, uint32_t m_tiles_all, uint32_t L, Tile& t) {
+__device__ __forceinline__ void decode_tile(const GemmParams& p, uint32_t m_tiles_all, uint32_t L, Tile& t, uint32_t g_from = 0) {
     if (p.row_off != nullptr) {
-        // find g with tile_pref[g]*w_tiles <= L < tile_pref[g+1]*w_tiles
-        uint32_t lo = 0, hi = p.groups;
+        // find g with tile_pref[g]*w_tiles <= L < tile_pref[g+1]*w_tiles.  A workgroup's next tile mostly lies in the
+        // same group or one of the next two: three independent loads settle that before the bisection's
+        // chain of dependent ones
+        const uint32_t G = p.groups;
+        uint32_t lo = g_from, hi = G;
+        const uint32_t i2 = lo + 2 < G ? lo + 2 : G, i3 = lo + 3 < G ? lo + 3 : G;
+        const uint32_t t1 = (uint32_t)p.tile_pref[lo + 1] * p.w_tiles, t2 = (uint32_t)p.tile_pref[i2] * p.w_tiles,
+                       t3 = (uint32_t)p.tile_pref[i3] * p.w_tiles;
+        if (t1 > L) hi = lo + 1;
+        else if (t2 > L) { lo += 1; hi = lo + 1; }
+        else if (t3 > L) { lo += 2; hi = lo + 1; }
+        else lo += 3;
         while (hi - lo > 1) {
             const uint32_t mid = (lo + hi) >> 1;
             if ((uint32_t)p.tile_pref[mid] * p.w_tiles <= L) lo = mid; else hi = mid;

@@ -179,8 +179,8 @@ __global__ __launch_bounds__(256) void mx_gemm_pipe_kernel(const GemmParams p) {
         r[3] = 0x00020000;
         return r;
     };
-    auto aim_loads_at = [&](uint32_t L) {
-        decode_tile<TM>(p, m_tiles_all, L, tq);
+    auto aim_loads_at = [&](uint32_t L, uint32_t g_from) {
+        decode_tile<TM>(p, m_tiles_all, L, tq, g_from);
         const uint32_t g = __builtin_amdgcn_readfirstlane(tq.g), wt = __builtin_amdgcn_readfirstlane(tq.wt);
         const uint32_t row0 = __builtin_amdgcn_readfirstlane(tq.row0);
         const uint32_t rows_valid = __builtin_amdgcn_readfirstlane(tq.rows_valid);
@@ -218,7 +218,7 @@ __global__ __launch_bounds__(256) void mx_gemm_pipe_kernel(const GemmParams p) {
         sgoff_w = wrow_of(64 * wave + lane) * p.ld_ws;
         sgoff_a = arow_of(64 * sa_blk + lane) * p.ld_as;
     };
-    aim_loads_at(tile_id);
+    aim_loads_at(tile_id, 0);
     Tile tc = tq;                               // tile of the MFMA stream / epilogue
 
     auto nslab_of = [](const GemmParams& q) -> uint32_t { return q.kbytes / kSlabBytes; };
@@ -562,7 +562,7 @@ __global__ __launch_bounds__(256) void mx_gemm_pipe_kernel(const GemmParams p) {
                 }
                 next_ok = next_id < run_end;
                 if (next_ok) {
-                    aim_loads_at(next_id);
+                    aim_loads_at(next_id, tq.g);      // tile ids only grow
                     sq = 0;
                 }
             }
