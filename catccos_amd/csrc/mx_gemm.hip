@@ -33,9 +33,13 @@ constexpr int kSlabBytes = 128;     // K bytes per LDS slab and row
 constexpr int kChunks = kSlabBytes / 16;
 constexpr int kXcds = 8;
 
-// kEpiStore16: bf16 or fp16 output whose rows and row pitch are multiples of four elements (one 8-byte store per
-// accumulator quad, no per-element edge handling): small enough to sit inside a persistent kernel's tile loop
-enum Epilogue { kEpiStore = 0, kEpiSwigluQuant = 1, kEpiStore16 = 2, kEpiI8DequantSwiglu = 3 };
+// kEpiStoreBf16 / kEpiStoreFp16: 16-bit output whose rows and row pitch are multiples of four elements (one 8-byte
+// store per accumulator quad, no per-element edge handling): small enough to sit inside a persistent kernel's tile
+// loop.  Two epilogues, not one with a run-time switch: a second copy of the store loop inside the kernel costs
+// registers, and values spilled because of it are reloaded inside the scheduled loop, where the waits that the
+// compiler puts behind such reloads drain the operand loads in flight.
+enum Epilogue { kEpiStore = 0, kEpiSwigluQuant = 1, kEpiStoreBf16 = 2, kEpiI8DequantSwiglu = 3, kEpiStoreFp16 = 4 };
+constexpr bool epi_is_lean_store(int epi) { return epi == kEpiStoreBf16 || epi == kEpiStoreFp16; }
 // epilogues whose weight tile pairs gate rows (first half of N) with their up partners (second half)
 constexpr bool epi_pairs_gate_up(int epi) { return epi == kEpiSwigluQuant || epi == kEpiI8DequantSwiglu; }
 // element "format" of the INT8 path inside the kernel templates (the public format codes are the MX ones)
@@ -220,37 +224,32 @@ __device__ __forceinline__ void epilogue(const GemmParams& p, const Tile& tc, v1
     const uint32_t l32 = lane & 31u, lh = lane >> 5;
     const uint32_t wt = tc.wt, row0 = tc.row0, rows_valid = tc.rows_valid;
     auto wfrag_row = [&](int f) -> uint32_t { return wfrag_row_of<TW, WW, EPI, FW>(ww, f); };
-    if constexpr (EPI == kEpiStore16) {
+    if constexpr (epi_is_lean_store(EPI)) {
         uint16_t* const c = reinterpret_cast<uint16_t*>(p.c);
-        auto store_all = [&](auto f16_c) {
-            constexpr bool kF16 = decltype(f16_c)::value;
-            auto pack = [](float a, float b) -> uint32_t {
-                if constexpr (kF16) {
-                    typedef _Float16 v2h __attribute__((ext_vector_type(2)));
-                    return __builtin_bit_cast(uint32_t, (v2h){(_Float16)a, (_Float16)b});
-                } else {
-                    return cvt_pk_bf16(a, b);
-                }
-            };
-#pragma unroll
-            for (int fm = 0; fm < FM; ++fm) {
-                const uint32_t mloc = wm * (TM / WM) + fm * 32 + l32;
-                if (mloc >= rows_valid) continue;
-                uint16_t* const crow = c + (size_t)(row0 + mloc) * p.ldc;
-#pragma unroll
-                for (int fw = 0; fw < FW; ++fw) {
-#pragma unroll
-                    for (int q = 0; q < 4; ++q) {
-                        const uint32_t ncol = wt * TW + wfrag_row(fw) + 8 * q + 4 * lh;
-                        if (ncol < p.n)
-                            *reinterpret_cast<uint2*>(crow + ncol) = make_uint2(pack(acc[fw][fm][4 * q], acc[fw][fm][4 * q + 1]),
-                                                                                pack(acc[fw][fm][4 * q + 2], acc[fw][fm][4 * q + 3]));
-                    }
-                }
+        auto pack = [](float a, float b) -> uint32_t {
+            if constexpr (EPI == kEpiStoreFp16) {
+                typedef _Float16 v2h __attribute__((ext_vector_type(2)));
+                return __builtin_bit_cast(uint32_t, (v2h){(_Float16)a, (_Float16)b});
+            } else {
+                return cvt_pk_bf16(a, b);
             }
         };
-        if (p.out_type == CMX_OUT_FP16) store_all(std::true_type{});
-        else store_all(std::false_type{});
+#pragma unroll
+        for (int fm = 0; fm < FM; ++fm) {
+            const uint32_t mloc = wm * (TM / WM) + fm * 32 + l32;
+            if (mloc >= rows_valid) continue;
+            uint16_t* const crow = c + (size_t)(row0 + mloc) * p.ldc;
+#pragma unroll
+            for (int fw = 0; fw < FW; ++fw) {
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    const uint32_t ncol = wt * TW + wfrag_row(fw) + 8 * q + 4 * lh;
+                    if (ncol < p.n)
+                        *reinterpret_cast<uint2*>(crow + ncol) = make_uint2(pack(acc[fw][fm][4 * q], acc[fw][fm][4 * q + 1]),
+                                                                            pack(acc[fw][fm][4 * q + 2], acc[fw][fm][4 * q + 3]));
+                }
+            }
+        }
     } else if constexpr (EPI == kEpiStore) {
 #pragma unroll
         for (int fm = 0; fm < FM; ++fm) {
@@ -1085,12 +1084,13 @@ int launch_tile(const GemmParams& p, int waves, uint32_t max_m_tiles, hipStream_
         // whole four-slab scale blocks, fetched 16 bytes per row: K a multiple of 512 bytes, 16-byte aligned scale rows
         if ((waves == 4 || waves == 5) && stream_ok && p.scale_vec16 && p.kbytes % (4 * kSlabBytes) == 0) {
             // plain 16-bit output with 4-element-aligned rows takes the lean store epilogue and with it the persistent kernel
-            constexpr int kLean = EPI == kEpiStore ? kEpiStore16 : EPI;
+            constexpr int kLeanBf16 = EPI == kEpiStore ? kEpiStoreBf16 : EPI, kLeanFp16 = EPI == kEpiStore ? kEpiStoreFp16 : EPI;
             const bool lean = EPI == kEpiStore && p.out_type != CMX_OUT_FP32 && p.n % 4 == 0 && p.ldc % 4 == 0 &&
                               (reinterpret_cast<uintptr_t>(p.c) & 7u) == 0;
             // (the 4 x 1 layout with the lean store epilogue does not fit the register file without spilling
             // inside the loop, so the persistent store kernel is always 2 x 2)
-            if (lean) return launch_gemm_pipe<FMT, kLean, 256, 2, 2, 2>(p, max_m_tiles, s);
+            if (lean && p.out_type == CMX_OUT_BF16) return launch_gemm_pipe<FMT, kLeanBf16, 256, 2, 2, 2>(p, max_m_tiles, s);
+            if (lean) return launch_gemm_pipe<FMT, kLeanFp16, 256, 2, 2, 2>(p, max_m_tiles, s);
             if (waves == 4) return launch_gemm_pipe<FMT, EPI, 256, 2, 2, 2>(p, max_m_tiles, s);
             return launch_gemm_pipe<FMT, EPI, 256, 4, 1, 2>(p, max_m_tiles, s);
         }
@@ -1102,7 +1102,8 @@ int launch_tile(const GemmParams& p, int waves, uint32_t max_m_tiles, hipStream_
                 // plain 16-bit output with 4-element-aligned rows: lean store epilogue, persistent kernel
                 const bool lean = p.out_type != CMX_OUT_FP32 && p.n % 4 == 0 && p.ldc % 4 == 0 && (reinterpret_cast<uintptr_t>(p.c) & 7u) == 0;
                 // (as with the 8-bit kernel the 4 x 1 layout would spill inside the loop: the persistent kernel is 2 x 2)
-                if (lean) return launch_gemm_pipe_fp4<kEpiStore16, 2, 2>(p, max_m_tiles, s);
+                if (lean && p.out_type == CMX_OUT_BF16) return launch_gemm_pipe_fp4<kEpiStoreBf16, 2, 2>(p, max_m_tiles, s);
+                if (lean) return launch_gemm_pipe_fp4<kEpiStoreFp16, 2, 2>(p, max_m_tiles, s);
                 if (waves == 4) return launch_gemm_pipe_fp4<EPI, 2, 2>(p, max_m_tiles, s);
                 return launch_gemm_pipe_fp4<EPI, 4, 1>(p, max_m_tiles, s);
             }
