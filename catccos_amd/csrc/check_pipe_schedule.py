@@ -14,7 +14,7 @@ For every instantiation that the library dispatches to, this script compiles tha
 (device only, nothing is linked or run) and reports the spills and waits found between the first and the last
 MFMA.  Run it after any change to the kernels, the epilogues or their helpers:
 
-    python3 catccos_amd/csrc/check_pipe_schedule.py          # about a minute per kernel
+    python3 catccos_amd/csrc/check_pipe_schedule.py          # a few seconds per kernel
 
 Exit status 0 when every kernel is clean.
 """

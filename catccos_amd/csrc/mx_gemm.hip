@@ -1306,8 +1306,9 @@ extern "C" int cmx_int8_gmm_dequant_swiglu(const int8_t* a, uint32_t lda, const 
     p.tile_ctr = tile_ctr;
     p.groups = groups;
     p.w_tiles = ceil_div(n / 2, kTile / 2);
-    // (a hand-scheduled variant of this kernel -- two i8 MFMAs per step and accumulator, issued in interleaved pairs --
-    // was measured at 997 us against 972 us for this one at 16 x 2048 x 7168 x 4096 and is not kept)
+    // (hand-scheduled variants of this kernel were measured twice at 16 x 2048 x 7168 x 4096 and are not kept: two i8
+    // MFMAs per step and accumulator in the 8-bit schedule 997 us, one per 32-K step in the 16-byte-fragment
+    // schedule shared with FP4, one tile per workgroup, 994-1000 us, against 967-975 us for this one)
     return launch_gemm_dl<kFmtI8, kTile, kTile, 2, 4, kEpiI8DequantSwiglu>(p, m_total / kTile + groups, s);
 }
 
