@@ -130,8 +130,8 @@ def main() -> int:
                 "achieved": flop / kern / 1e12, "peak": MXFP8_PEAK_TFLOPS, "unit": "TFLOP/s",
                 "frac": flop / kern / 1e12 / MXFP8_PEAK_TFLOPS,
                 # HBM-side bytes per launch from the rocprofv3 --pmc runs summarised under profiles/
-                # (FETCH_SIZE 1 177 361 KiB x 2.0 + WRITE_SIZE 150 521 KiB x 1.0, factors from a 1 GiB copy)
-                "traffic": 1177361 * 1024 * 2.0 + 150521 * 1024 * 1.0,
+                # (FETCH_SIZE 1 151 590 KiB x 2.0 + WRITE_SIZE 118 695 KiB x 1.0, factors from a 1 GiB copy)
+                "traffic": 1151590 * 1024 * 2.0 + 118695 * 1024 * 1.0,
                 "flop_per_launch": flop, "avg_launch_us": kern * 1e6}
 
     # ------------------------------------------------------------------ CPU baseline -----------
