@@ -10,6 +10,10 @@ add are fatal for the schedule and invisible in the source:
   behind every reload of a spilled value, also when the reload sits before the loop and the first use inside it,
   and such a wait drains the operand loads that the schedule keeps in flight.
 
+A third check concerns correctness: an LDS-DMA load (``buffer_load ... lds``) takes its LDS address from M0, and the
+kernels that issue it in two statements (write of M0, a scheduled instruction in the wait state, the load) rely on
+nothing else writing M0 in between and on at least one instruction standing there.
+
 For every instantiation that the library dispatches to, this script compiles that one kernel to assembly
 (device only, nothing is linked or run) and reports the spills and waits found between the first and the last
 MFMA.  Run it after any change to the kernels, the epilogues or their helpers:
@@ -72,6 +76,16 @@ def check(kernel: str, own_waits: set[int], workdir: str) -> list[str]:
     if not mfma:
         return ["no MFMA found"]
     problems = []
+    code = [ln for ln in lines if ln and not ln.startswith(";")]
+    for i, ln in enumerate(code):
+        if ln.startswith("buffer_load") and ln.endswith(" lds"):
+            j = i - 1
+            while j >= 0 and not re.search(r"\bm0\b", code[j]):
+                j -= 1
+            between = [x for x in code[j + 1: i] if not x.endswith(":")]
+            labels = [x for x in code[j + 1: i] if x.endswith(":") and not x.startswith(".Lskip")]      # the MFMA-skip branches are local
+            if j < 0 or not code[j].startswith("s_mov_b32 m0") or not between or labels:
+                problems.append("LDS-DMA load without its own M0 write and wait state: " + ln)
     for ln in lines[mfma[0]: mfma[-1] + 1]:
         if ln.startswith("scratch_"):
             problems.append("spill traffic inside the scheduled stream: " + ln)
