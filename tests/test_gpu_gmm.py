@@ -71,7 +71,7 @@ def test_gmm_many_ragged_groups_every_row(tile):
     assert np.array_equal(host(scales), ws2) and np.array_equal(host(codes), wq2)
 
 
-@pytest.mark.parametrize("fmt,k", [("E4M3", 512), ("E2M1", 512), ("E2M1", 1024)])
+@pytest.mark.parametrize("fmt,k", [("E4M3", 512), ("E4M3", 1536), ("E2M1", 512), ("E2M1", 1024), ("E2M1", 1536)])
 def test_more_tiles_than_workgroups_every_row(fmt, k):
     """Enough tiles (about 300 of 256 x 256) that the persistent kernels, one workgroup per CU, walk on to a second
     tile: the load stream crosses the tile boundary, the next tile comes from the per-XCD counters, and every
