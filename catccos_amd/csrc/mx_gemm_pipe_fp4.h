@@ -4,18 +4,25 @@
 // A 128-byte K slab holds 256 FP4 elements = four MFMA steps of 64 K; a lane's fragment of one step is a
 // single 16-byte run (the 32-element MX block of its half-wave), and a slab carries two scale dwords per
 // row.  As in the 8-bit two-slot kernels the scales arrive 16 bytes per row at a time -- here the scales of two
-// slabs -- into a ring of two such blocks, [block][row][4 dwords].  An FP4 MFMA takes 8 passes (32 clocks), so a slab is again 64 x 32 = 2048 MFMA clocks per wavefront
-// for the same 64 KiB of loads as in the 8-bit kernel.  Four wavefronts in a 2 x 2 grid, 16 accumulator
-// tiles in AGPRs, two fragment sets of 8 x 4 VGPRs.  Per slab s (ring slot s%2):
-//   step 0, 1: 16 MFMAs each; behind the first 8 the 8 reads of the next step's fragments (same slot);
-//   step 2:    likewise (reads of step 3); after MFMA 9 those have landed and the slot is never read again:
-//              barrier, then the first 6 tile loads of slab s+2 behind the remaining MFMAs; the step ends with
-//              the wait for the own loads of slab s+1 and the barrier that publishes it;
-//   step 3:    the other 10 tile loads of slab s+2 (and, every second slab, the next scale block), the reads of
-//              step 0 of slab s+1 from the other slot, its 16 scale dwords and their per-half-wave byte shift.
-// With the lean 16-bit store epilogue the kernel is persistent like its 8-bit counterpart: one workgroup per CU walks
-// the tiles of its XCD's run and carries the load stream across tile boundaries, so that the first slabs of a tile
-// arrive while the previous tile's epilogue runs.  With the general store epilogue it takes one tile per workgroup.
+// slabs -- into a ring of two such blocks, [block][row][4 dwords].  An FP4 MFMA takes 8 passes (32 clocks), so a
+// slab is again 64 x 32 = 2048 MFMA clocks per wavefront for the same 64 KiB of loads as in the 8-bit kernel, but
+// an MFMA leaves room for only about six other instructions: the instruction stream is kept thin (a load's M0
+// write and the load itself stand on either side of an MFMA instead of an s_nop, both scale dwords of a row come
+// with one 8-byte read, the byte shifts are spread over a step).  Four wavefronts, 16 accumulator tiles in AGPRs,
+// two fragment sets of NF x 4 VGPRs.  Per slab s (ring slot s%2):
+//   step 0:    16 MFMAs; behind the first NF the reads of step 1's fragments, behind the others the scale reads
+//              of slab s+1 (its block landed long ago);
+//   step 1:    behind the first NF MFMAs the reads of step 2's fragments, behind the others the per-half-wave
+//              byte shifts of those scales into the other scale set;
+//   step 2:    reads of step 3; after MFMA 9 they have landed and the slot is never read again: barrier, then the
+//              first 6 tile loads of slab s+2 around the remaining MFMAs; the step ends with the wait for the own
+//              loads of slab s+1 and the barrier that publishes it;
+//   step 3:    the other 10 tile loads of slab s+2 (and, every second slab, the next scale block) and the reads of
+//              step 0 of slab s+1 from the other slot.
+// With the lean 16-bit store epilogues the kernel is persistent like its 8-bit counterpart: one workgroup per CU
+// walks the tiles of its XCD's run and carries the load stream across tile boundaries, so that the first slabs of
+// a tile arrive while the previous tile's epilogue runs.  With the general store epilogue it takes one tile per
+// workgroup.
 #pragma once
 
 // An LDS-DMA load in two statements, so that a scheduled instruction (an MFMA, an LDS read) can stand where the wait
