@@ -33,9 +33,8 @@ constexpr int kSlabBytes = 128;     // K bytes per LDS slab and row
 constexpr int kChunks = kSlabBytes / 16;
 constexpr int kXcds = 8;
 
-// kEpiStoreBf16 / kEpiStoreFp16: 16-bit output whose rows and row pitch are multiples of four elements (one 8-byte
-// store per accumulator quad, no per-element edge handling): small enough to sit inside a persistent kernel's tile
-// loop.  Two epilogues, not one with a run-time switch: a second copy of the store loop inside the kernel costs
+// kEpiStoreBf16 / kEpiStoreFp16: 16-bit output whose rows and row pitch are multiples of eight elements (16-byte
+// stores, no per-element edge handling): small enough to sit inside a persistent kernel's tile loop.  Two epilogues, not one with a run-time switch: a second copy of the store loop inside the kernel costs
 // registers, and values spilled because of it are reloaded inside the scheduled loop, where the waits that the
 // compiler puts behind such reloads drain the operand loads in flight.
 enum Epilogue { kEpiStore = 0, kEpiSwigluQuant = 1, kEpiStoreBf16 = 2, kEpiI8DequantSwiglu = 3, kEpiStoreFp16 = 4 };
@@ -237,16 +236,26 @@ __device__ __forceinline__ void epilogue(const GemmParams& p, const Tile& tc, v1
 #pragma unroll
         for (int fm = 0; fm < FM; ++fm) {
             const uint32_t mloc = wm * (TM / WM) + fm * 32 + l32;
-            if (mloc >= rows_valid) continue;
-            uint16_t* const crow = c + (size_t)(row0 + mloc) * p.ldc;
+            const bool mvalid = mloc < rows_valid;
+            uint16_t* const crow = c + (size_t)(row0 + (mvalid ? mloc : 0)) * p.ldc;
 #pragma unroll
             for (int fw = 0; fw < FW; ++fw) {
+                // A lane holds columns 8q + 4 lh + {0..3} of its row for q = 0..3, its partner in the other half-wave
+                // (same row) the four next to them.  Swapping register halves between the two gives either lane eight
+                // consecutive columns: one 16-byte store instead of two 8-byte ones.
 #pragma unroll
-                for (int q = 0; q < 4; ++q) {
-                    const uint32_t ncol = wt * TW + wfrag_row(fw) + 8 * q + 4 * lh;
-                    if (ncol < p.n)
-                        *reinterpret_cast<uint2*>(crow + ncol) = make_uint2(pack(acc[fw][fm][4 * q], acc[fw][fm][4 * q + 1]),
-                                                                            pack(acc[fw][fm][4 * q + 2], acc[fw][fm][4 * q + 3]));
+                for (int qp = 0; qp < 2; ++qp) {
+                    const int q = 2 * qp;
+                    const uint32_t a0 = pack(acc[fw][fm][4 * q], acc[fw][fm][4 * q + 1]);
+                    const uint32_t a1 = pack(acc[fw][fm][4 * q + 2], acc[fw][fm][4 * q + 3]);
+                    const uint32_t b0 = pack(acc[fw][fm][4 * q + 4], acc[fw][fm][4 * q + 5]);
+                    const uint32_t b1 = pack(acc[fw][fm][4 * q + 6], acc[fw][fm][4 * q + 7]);
+                    // upper half of a <-> lower half of b: lower lanes end up with columns 8q .. 8q+7 in (a, b), upper
+                    // lanes with 8(q+1) .. 8(q+1)+7
+                    const auto s0 = __builtin_amdgcn_permlane32_swap(a0, b0, false, false);
+                    const auto s1 = __builtin_amdgcn_permlane32_swap(a1, b1, false, false);
+                    const uint32_t ncol = wt * TW + wfrag_row(fw) + 8 * (q + lh);
+                    if (mvalid && ncol < p.n) *reinterpret_cast<uint4*>(crow + ncol) = make_uint4(s0[0], s1[0], s0[1], s1[1]);
                 }
             }
         }
@@ -1083,10 +1092,10 @@ int launch_tile(const GemmParams& p, int waves, uint32_t max_m_tiles, hipStream_
     if constexpr (TW == 256 && TM == 256 && FMT != CMX_FMT_E2M1) {
         // whole four-slab scale blocks, fetched 16 bytes per row: K a multiple of 512 bytes, 16-byte aligned scale rows
         if ((waves == 4 || waves == 5) && stream_ok && p.scale_vec16 && p.kbytes % (4 * kSlabBytes) == 0) {
-            // plain 16-bit output with 4-element-aligned rows takes the lean store epilogue and with it the persistent kernel
+            // plain 16-bit output with 8-element-aligned rows takes the lean store epilogue and with it the persistent kernel
             constexpr int kLeanBf16 = EPI == kEpiStore ? kEpiStoreBf16 : EPI, kLeanFp16 = EPI == kEpiStore ? kEpiStoreFp16 : EPI;
-            const bool lean = EPI == kEpiStore && p.out_type != CMX_OUT_FP32 && p.n % 4 == 0 && p.ldc % 4 == 0 &&
-                              (reinterpret_cast<uintptr_t>(p.c) & 7u) == 0;
+            const bool lean = EPI == kEpiStore && p.out_type != CMX_OUT_FP32 && p.n % 8 == 0 && p.ldc % 8 == 0 &&
+                              (reinterpret_cast<uintptr_t>(p.c) & 15u) == 0;
             // (the 4 x 1 layout with the lean store epilogue does not fit the register file without spilling
             // inside the loop, so the persistent store kernel is always 2 x 2)
             if (lean && p.out_type == CMX_OUT_BF16) return launch_gemm_pipe<FMT, kLeanBf16, 256, 2, 2, 2>(p, max_m_tiles, s);
@@ -1099,8 +1108,8 @@ int launch_tile(const GemmParams& p, int waves, uint32_t max_m_tiles, hipStream_
         // hand-scheduled FP4 kernel: whole two-slab scale blocks (K a multiple of 512 elements), 16-byte aligned scale rows
         if ((waves == 4 || waves == 5) && stream_ok && p.scale_vec16 && p.kbytes % (2 * kSlabBytes) == 0) {
             if constexpr (EPI == kEpiStore) {
-                // plain 16-bit output with 4-element-aligned rows: lean store epilogue, persistent kernel
-                const bool lean = p.out_type != CMX_OUT_FP32 && p.n % 4 == 0 && p.ldc % 4 == 0 && (reinterpret_cast<uintptr_t>(p.c) & 7u) == 0;
+                // plain 16-bit output with 8-element-aligned rows: lean store epilogue, persistent kernel
+                const bool lean = p.out_type != CMX_OUT_FP32 && p.n % 8 == 0 && p.ldc % 8 == 0 && (reinterpret_cast<uintptr_t>(p.c) & 15u) == 0;
                 // (as with the 8-bit kernel the 4 x 1 layout would spill inside the loop: the persistent kernel is 2 x 2)
                 if (lean && p.out_type == CMX_OUT_BF16) return launch_gemm_pipe_fp4<kEpiStoreBf16, 2, 2>(p, max_m_tiles, s);
                 if (lean) return launch_gemm_pipe_fp4<kEpiStoreFp16, 2, 2>(p, max_m_tiles, s);
