@@ -1110,9 +1110,11 @@ int launch_tile(const GemmParams& p, int waves, uint32_t max_m_tiles, hipStream_
             if constexpr (EPI == kEpiStore) {
                 // plain 16-bit output with 8-element-aligned rows: lean store epilogue, persistent kernel
                 const bool lean = p.out_type != CMX_OUT_FP32 && p.n % 8 == 0 && p.ldc % 8 == 0 && (reinterpret_cast<uintptr_t>(p.c) & 15u) == 0;
-                // (as with the 8-bit kernel the 4 x 1 layout would spill inside the loop: the persistent kernel is 2 x 2)
-                if (lean && p.out_type == CMX_OUT_BF16) return launch_gemm_pipe_fp4<kEpiStoreBf16, 2, 2>(p, max_m_tiles, s);
-                if (lean) return launch_gemm_pipe_fp4<kEpiStoreFp16, 2, 2>(p, max_m_tiles, s);
+                // (unlike the 8-bit kernel, whose fragments take twice the registers, the 4 x 1 layout fits here too)
+                if (lean && waves == 4 && p.out_type == CMX_OUT_BF16) return launch_gemm_pipe_fp4<kEpiStoreBf16, 2, 2>(p, max_m_tiles, s);
+                if (lean && waves == 4) return launch_gemm_pipe_fp4<kEpiStoreFp16, 2, 2>(p, max_m_tiles, s);
+                if (lean && p.out_type == CMX_OUT_BF16) return launch_gemm_pipe_fp4<kEpiStoreBf16, 4, 1>(p, max_m_tiles, s);
+                if (lean) return launch_gemm_pipe_fp4<kEpiStoreFp16, 4, 1>(p, max_m_tiles, s);
                 if (waves == 4) return launch_gemm_pipe_fp4<EPI, 2, 2>(p, max_m_tiles, s);
                 return launch_gemm_pipe_fp4<EPI, 4, 1>(p, max_m_tiles, s);
             }

@@ -71,13 +71,14 @@ def test_gmm_many_ragged_groups_every_row(tile):
     assert np.array_equal(host(scales), ws2) and np.array_equal(host(codes), wq2)
 
 
-@pytest.mark.parametrize("fmt,k", [("E4M3", 512), ("E4M3", 1536), ("E2M1", 512), ("E2M1", 1024), ("E2M1", 1536)])
-def test_more_tiles_than_workgroups_every_row(fmt, k):
+@pytest.mark.parametrize("fmt,k,waves", [("E4M3", 512, 4), ("E4M3", 1536, 4), ("E2M1", 512, 4), ("E2M1", 1024, 4), ("E2M1", 1536, 4),
+                                         ("E2M1", 512, 5), ("E2M1", 1536, 5)])
+def test_more_tiles_than_workgroups_every_row(fmt, k, waves):
     """Enough tiles (about 300 of 256 x 256) that the persistent kernels, one workgroup per CU, walk on to a second
     tile: the load stream crosses the tile boundary, the next tile comes from the per-XCD counters, and every
     row of every group must still come out right, with the rows past the groups untouched."""
     from catccos_amd import ops, _lib
-    _lib.load().cmx_debug_force_tile(256, 256, 4)
+    _lib.load().cmx_debug_force_tile(256, 256, waves)
     rng = np.random.default_rng(91)
     counts = [int(c) for c in rng.integers(0, 700, size=36)] + [256, 512, 0, 128, 1, 255]
     n = 1024
