@@ -37,11 +37,13 @@ FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-Xclang", "-target-featu
          f"-I{os.path.join(ROOT, 'include')}", f"-I{HERE}", "-S", "--cuda-device-only", "-Wno-unused-command-line-argument"]
 
 # (explicit instantiation, the schedule's own vmcnt waits inside the stream)
-#   mx_gemm_pipe_kernel<FMT, EPI, TM, WW, WM, NSLOT>; EPI 0 store, 1 SwiGLU + requant, 2 lean bf16, 4 lean fp16
+#   mx_gemm_pipe_kernel<FMT, EPI, TM, WW, WM, NSLOT>; EPI 0 store, 1 SwiGLU + requant, 2 lean bf16, 4 lean fp16, 5 = 1 + bf16 activations
 #   mx_gemm_pipe_fp4_kernel<EPI, WW, WM>
 KERNELS = [
     ("mx_gemm_pipe_kernel<0, 1, 256, 2, 2, 2>", {7}),
     ("mx_gemm_pipe_kernel<0, 1, 256, 4, 1, 2>", {8}),
+    ("mx_gemm_pipe_kernel<0, 5, 256, 2, 2, 2>", {7}),          # SwiGLU + requant that also writes the bf16 activations
+    ("mx_gemm_pipe_kernel<0, 5, 256, 4, 1, 2>", {8}),
     ("mx_gemm_pipe_kernel<0, 2, 256, 2, 2, 2>", {7}),
     ("mx_gemm_pipe_kernel<0, 4, 256, 2, 2, 2>", {7}),
     ("mx_gemm_pipe_kernel<0, 0, 256, 2, 2, 2>", {7}),

@@ -37,10 +37,14 @@ constexpr int kXcds = 8;
 // stores, no per-element edge handling): small enough to sit inside a persistent kernel's tile loop.  Two epilogues, not one with a run-time switch: a second copy of the store loop inside the kernel costs
 // registers, and values spilled because of it are reloaded inside the scheduled loop, where the waits that the
 // compiler puts behind such reloads drain the operand loads in flight.
-enum Epilogue { kEpiStore = 0, kEpiSwigluQuant = 1, kEpiStoreBf16 = 2, kEpiI8DequantSwiglu = 3, kEpiStoreFp16 = 4 };
+// kEpiSwigluQuantAct: kEpiSwigluQuant that also writes the bf16 SwiGLU output (what the tests check the requantised
+// codes against).  A kernel of its own for the same reason: the extra output path costs the SwiGLU kernels
+// 30 registers, all of them spilled at the tile boundaries, 3 % of a launch, whether the output is asked for or not.
+enum Epilogue { kEpiStore = 0, kEpiSwigluQuant = 1, kEpiStoreBf16 = 2, kEpiI8DequantSwiglu = 3, kEpiStoreFp16 = 4, kEpiSwigluQuantAct = 5 };
 constexpr bool epi_is_lean_store(int epi) { return epi == kEpiStoreBf16 || epi == kEpiStoreFp16; }
+constexpr bool epi_is_swiglu_quant(int epi) { return epi == kEpiSwigluQuant || epi == kEpiSwigluQuantAct; }
 // epilogues whose weight tile pairs gate rows (first half of N) with their up partners (second half)
-constexpr bool epi_pairs_gate_up(int epi) { return epi == kEpiSwigluQuant || epi == kEpiI8DequantSwiglu; }
+constexpr bool epi_pairs_gate_up(int epi) { return epi_is_swiglu_quant(epi) || epi == kEpiI8DequantSwiglu; }
 // element "format" of the INT8 path inside the kernel templates (the public format codes are the MX ones)
 constexpr int kFmtI8 = 8;
 
@@ -379,11 +383,13 @@ __device__ __forceinline__ void epilogue(const GemmParams& p, const Tile& tc, v1
                     pk[j] = cvt_pk_bf16(a0, a1);
                     m = pk_max_u16(m, pk[j] & 0x7FFF7FFFu);
                 }
-                if (p.act_bf16 && mvalid) {
+                if constexpr (EPI == kEpiSwigluQuantAct) {
+                    if (p.act_bf16 && mvalid) {
 #pragma unroll
-                    for (int r = 0; r < 16; ++r) {
-                        const uint32_t ncol = ncol0 + 8 * (r >> 2) + 4 * lh + (r & 3);
-                        if (ncol < half) p.act_bf16[mrow * half + ncol] = (uint16_t)(pk[r >> 1] >> (16 * (r & 1)));
+                        for (int r = 0; r < 16; ++r) {
+                            const uint32_t ncol = ncol0 + 8 * (r >> 2) + 4 * lh + (r & 3);
+                            if (ncol < half) p.act_bf16[mrow * half + ncol] = (uint16_t)(pk[r >> 1] >> (16 * (r & 1)));
+                        }
                     }
                 }
                 uint32_t amax = max(m & 0xFFFFu, m >> 16);
@@ -1235,6 +1241,7 @@ int gmm_common(GemmParams& p, const int32_t* group_sizes, uint32_t groups, uint3
     p.groups = groups;
     p.w_tiles = swiglu ? ceil_div(p.n / 2, t.tw / 2) : ceil_div(p.n, t.tw);
     const uint32_t max_m_tiles = m_total / t.tm + groups;
+    if (swiglu && p.act_bf16 != nullptr) return dispatch_tile<CMX_FMT_E4M3, kEpiSwigluQuantAct>(p, t, max_m_tiles, s);
     if (swiglu) return dispatch_tile<CMX_FMT_E4M3, kEpiSwigluQuant>(p, t, max_m_tiles, s);
     switch (fmt) {
         case CMX_FMT_E4M3: return dispatch_tile<CMX_FMT_E4M3, kEpiStore>(p, t, max_m_tiles, s);

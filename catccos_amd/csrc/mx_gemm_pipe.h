@@ -193,7 +193,7 @@ __global__ __launch_bounds__(256) void mx_gemm_pipe_kernel(const GemmParams p) {
         // global row of tile row r (rows past the edge re-read the last valid row; their results are never stored)
         auto wrow_of = [&](uint32_t r) -> uint32_t {
             uint32_t gr;
-            if (EPI == kEpiSwigluQuant) {
+            if (epi_is_swiglu_quant(EPI)) {
                 const uint32_t half = p.n >> 1;
                 uint32_t rr = r < TW / 2 ? wt * (TW / 2) + r : wt * (TW / 2) + (r - TW / 2);
                 rr = rr < half ? rr : half - 1;
@@ -254,7 +254,7 @@ __global__ __launch_bounds__(256) void mx_gemm_pipe_kernel(const GemmParams p) {
     // a lane reads 16-byte chunks lh, lh+2 (step 0) and lh+4, lh+6 (step 1) of its row; all rows of a
     // lane share the low five bits l32, hence the swizzle term
     const uint32_t x = (l32 & 7u) ^ ((l32 >> 3) & 1u);
-    const uint32_t w_row_base = EPI == kEpiSwigluQuant ? ww * (TW / 2 / WW) : ww * (TW / WW);
+    const uint32_t w_row_base = epi_is_swiglu_quant(EPI) ? ww * (TW / 2 / WW) : ww * (TW / WW);
     uint32_t wb[NSLOT][4], ab[NSLOT][4];       // [slot][chunk j]
 #pragma unroll
     for (int s = 0; s < NSLOT; ++s)
@@ -287,7 +287,7 @@ __global__ __launch_bounds__(256) void mx_gemm_pipe_kernel(const GemmParams p) {
     uint32_t sraw[NF], scur[NSLOT][NF];      // shifted scales alternate between two sets: a set is rewritten one slab after its last use
 
     // weight fragment f sits f*32 rows (SwiGLU: the gate fragments, then their up partners 128 rows on) below the base
-#define CMX_PIPE_WOFF(f) ((EPI == kEpiSwigluQuant ? ((f) < FW / 2 ? (f) * 32 : TW / 2 + ((f) - FW / 2) * 32) : (f) * 32))
+#define CMX_PIPE_WOFF(f) ((epi_is_swiglu_quant(EPI) ? ((f) < FW / 2 ? (f) * 32 : TW / 2 + ((f) - FW / 2) * 32) : (f) * 32))
     // one 16-byte read: r = 2 * position in the read order + half (0: registers 0-3, 1: registers 4-7)
     auto read_half = [&](auto slot_c, auto step_c, auto r_c, v4i (&flo)[NF], v4i (&fhi)[NF]) {
         constexpr int slot = decltype(slot_c)::value, step = decltype(step_c)::value, r = decltype(r_c)::value;

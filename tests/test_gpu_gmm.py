@@ -119,6 +119,8 @@ def test_swiglu_requant_more_tiles_than_workgroups(waves):
     assert bad == 0, (bad, worst)
     wq2, ws2 = O.mx_quant_bf16(host(act), "E4M3", "rne")
     assert np.array_equal(host(scales), ws2) and np.array_equal(host(codes), wq2)
+    codes_p, scales_p = ops.mx_gmm_swiglu_quant(dev(aq), dev(asc), dev(wq), dev(ws), dev(np.array(counts, dtype=np.int32)), k)[:2]
+    assert torch.equal(codes_p, codes) and torch.equal(scales_p, scales)        # same without the bf16 output
 
 
 @pytest.mark.parametrize("tile", [None, (256, 128, 5), (128, 128, 4)])
@@ -223,6 +225,9 @@ def test_gmm1_swiglu_requant(tile):
     wq2, ws2 = O.mx_quant_bf16(act_bits, "E4M3", "rne")
     assert np.array_equal(host(scales), ws2)
     assert np.array_equal(host(codes), wq2)
+    # the kernels that do not write the bf16 activations (separate instantiations) produce the same codes and scales
+    codes_p, scales_p = ops.mx_gmm_swiglu_quant(dev(aq), dev(asc), dev(wq), dev(ws), dev(np.array(counts, dtype=np.int32)), k)[:2]
+    assert torch.equal(codes_p, codes) and torch.equal(scales_p, scales)
     # end to end the dequantised activations stay within tolerance of the golden's
     deq = O.mx_dequant(host(codes), host(scales))
     deq_g = O.mx_dequant(q_g, s_g)
