@@ -8,9 +8,13 @@ from __future__ import annotations
 import ctypes as C
 import os
 
+import sys
+
 _HERE = os.path.dirname(os.path.abspath(__file__))
-# CATCCOS_MX_LIB points at another build of the same library (e.g. an experimental kernel variant)
-LIB_PATH = os.environ.get("CATCCOS_MX_LIB") or os.path.join(_HERE, "lib", "libcatccos_mx.so")
+DEFAULT_LIB_PATH = os.path.join(_HERE, "lib", "libcatccos_mx.so")
+# CATCCOS_MX_LIB points at another build of the same library (e.g. an experimental kernel variant); load() says so
+# on stderr, so that no run uses a substitute unnoticed
+LIB_PATH = os.environ.get("CATCCOS_MX_LIB") or DEFAULT_LIB_PATH
 
 u8p, i32p, f32p, vp = C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p
 u32, i32, u64, sz = C.c_uint32, C.c_int, C.c_uint64, C.c_size_t
@@ -65,29 +69,42 @@ SIGNATURES = {
     "catccos_ascend950_dispatch_ffn_combine": (i32, [u32, vp, u64, u8p, u8p, u8p, u8p, u8p, u8p, u8p, u8p, u8p, u8p,
                                                      u32, u32, u32, u32, u32, i32]),
     "cmx_ffn_workspace_layout_get": (i32, [u32, u32, u32, u32, u32, C.POINTER(FfnWorkspaceLayout)]),
-    "cmx_mfma_raw_probe": (i32, [vp, vp, i32p, i32p, f32p, i32, i32, i32, vp]),
-    "cmx_debug_force_tile": (i32, [i32, i32, i32]),
-    "cmx_debug_disable_streaming": (i32, [i32]),
+    "cmx_init": (i32, []),
 }
 
 _lib = None
 
 
-def load() -> C.CDLL:
-    global _lib
-    if _lib is not None:
-        return _lib
-    if not os.path.exists(LIB_PATH):
+def bind(path: str, extra_signatures=None) -> C.CDLL:
+    """Loads the shared library at ``path`` and types every entry point of the C ABI (plus ``extra_signatures``)."""
+    if not os.path.exists(path):
         raise ImportError(
-            f"{LIB_PATH} is missing: build it with `python -m catccos_amd.build` (needs hipcc). "
+            f"{path} is missing: build it with `python -m catccos_amd.build` (needs hipcc). "
             "There is no CPU fallback.")
-    lib = C.CDLL(LIB_PATH)
-    for name, (res, args) in SIGNATURES.items():
+    lib = C.CDLL(path)
+    for name, (res, args) in {**SIGNATURES, **(extra_signatures or {})}.items():
         fn = getattr(lib, name)          # AttributeError names the missing symbol
         fn.restype = res
         fn.argtypes = args
-    _lib = lib
     return lib
+
+
+def load() -> C.CDLL:
+    """The library every function of the package calls."""
+    global _lib
+    if _lib is None:
+        if LIB_PATH != DEFAULT_LIB_PATH:
+            print(f"catccos_amd: CATCCOS_MX_LIB overrides the library: loading {LIB_PATH}", file=sys.stderr)
+        _lib = bind(LIB_PATH)
+    return _lib
+
+
+def activate(lib) -> "C.CDLL | None":
+    """Makes ``lib`` (a result of bind(), or None for the default) the library that load() returns; returns the
+    previous one.  The test suite uses it to run the package's front end on the test build of the library."""
+    global _lib
+    prev, _lib = _lib, lib
+    return prev
 
 
 class CmxError(RuntimeError):

@@ -43,6 +43,26 @@ def _filter(text: str) -> str:
     return "\n".join(keep)
 
 
+def compile_object(path: str, obj: str, extra_flags=(), verbose: bool = False) -> str:
+    """hipcc -c of one .hip file with the library's flags (plus ``extra_flags``)."""
+    cmd = [HIPCC, *FLAGS, *extra_flags, "-c", path, "-o", obj]
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    out = _filter(r.stdout + r.stderr)
+    if r.returncode != 0:
+        raise RuntimeError(f"hipcc failed on {path}:\n{out}")
+    if verbose and out:
+        print(out)
+    return obj
+
+
+def link_shared(lib: str, objs) -> str:
+    r = subprocess.run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", lib, *objs],
+                       capture_output=True, text=True)
+    if r.returncode != 0:
+        raise RuntimeError("link failed:\n" + _filter(r.stdout + r.stderr))
+    return lib
+
+
 def _compile(src: str, verbose: bool) -> str:
     obj = os.path.join(OBJ, src[:-4] + ".o")
     cmd = [HIPCC, *FLAGS, "-c", os.path.join(CSRC, src), "-o", obj]

@@ -83,6 +83,9 @@ extern "C" int catccos_ascend950_dispatch_ffn_combine(uint32_t blockDim, cmx_str
     CMX_REQUIRE(rankSize == 1, "one device only: rankSize must be 1");
     CMX_REQUIRE(x && expertIdx && gateWeight && w1 && w1Scale && w2 && w2Scale && out && workspace, "null pointer");
     CMX_REQUIRE(m > 0 && localExperts > 0 && topK > 0 && topK <= localExperts, "bad routing shape");
+    // limits of the stages further down the chain, checked before anything is launched
+    CMX_REQUIRE(topK <= 64, "topK must not exceed 64 (weighted combine)");
+    CMX_REQUIRE((uint64_t)m * topK < (1ull << 31), "m * topK must stay below 2^31 routes");
     CMX_REQUIRE(k % 256 == 0 && n % 512 == 0, "MXFP8 FFN requires K % 256 == 0 and N % 512 == 0");
     CMX_REQUIRE((reinterpret_cast<uintptr_t>(workspace) & 255u) == 0, "workspace must be 256-byte aligned");
     cmx_ffn_workspace_layout L;

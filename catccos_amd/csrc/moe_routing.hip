@@ -131,55 +131,148 @@ __global__ __launch_bounds__(64) void route_scatter_kernel(const int32_t* __rest
 
 // ---- fused quantise + scatter -------------------------------------------------------------------
 
-// Four lanes per MX block as in the plain quantizer; k % 32 == 0, rows 16-byte aligned.
+// Two lanes per MX block: each takes 16 elements with two 16-byte loads issued together, so a destination row is
+// written 16 bytes per lane, 1 KiB per wavefront and store instruction.  A workgroup owns 128 consecutive blocks.
+// The destination rows of the token are read before the arithmetic, eight at a time.  When scale rows hold whole
+// dwords (VEC_SCALES: k a multiple of 128, dword-aligned scale rows) the scale bytes of four neighbouring blocks
+// travel in one dword store instead of four byte stores.  k % 32 == 0, rows 16-byte aligned.
+template <bool VEC_SCALES>
 __global__ __launch_bounds__(256) void quant_scatter_kernel(const uint16_t* __restrict__ x, uint32_t ld_x,
                                                              const int32_t* __restrict__ src2sorted,
                                                              uint8_t* __restrict__ out_codes, uint32_t ld_out,
                                                              uint8_t* __restrict__ out_scales, uint32_t ld_outs,
                                                              uint32_t tokens, uint32_t k, uint32_t top_k, uint32_t nb,
                                                              uint32_t total_blocks) {
-    const uint32_t q = threadIdx.x & 3u;
-    const uint32_t b = blockIdx.x * 64 + (threadIdx.x >> 2);
+    const uint32_t h = threadIdx.x & 1u;
+    const uint32_t b = blockIdx.x * 128 + (threadIdx.x >> 1);
     const bool live = b < total_blocks;
     const uint32_t row = live ? b / nb : 0;
     const uint32_t kb = live ? b - row * nb : 0;
-    const uint32_t col = kb * 32 + q * 8;
-    uint4 raw = make_uint4(0, 0, 0, 0);
-    if (live) raw = *reinterpret_cast<const uint4*>(x + (size_t)row * ld_x + col);
-    // amax, clamp and cast on packed bf16 bit patterns, as in the stand-alone quantizer's fast path
-    const uint32_t d[4] = {raw.x, raw.y, raw.z, raw.w};
-    uint32_t a[4];
+    const uint32_t col = kb * 32 + h * 16;
+    uint4 raw0 = make_uint4(0, 0, 0, 0), raw1 = raw0;
+    if (live) {
+        const uint16_t* src = x + (size_t)row * ld_x + col;
+        raw0 = *reinterpret_cast<const uint4*>(src);
+        raw1 = *reinterpret_cast<const uint4*>(src + 8);
+    }
+    int32_t dst[8];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) a[i] = d[i] & 0x7FFF7FFFu;
-    uint32_t m = pk_max_u16(pk_max_u16(a[0], a[1]), pk_max_u16(a[2], a[3]));
-    m = pk_max_u16(m, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)m, 0xB1, 0xF, 0xF, true));
-    m = pk_max_u16(m, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)m, 0x4E, 0xF, 0xF, true));
+    for (int j = 0; j < 8; ++j) dst[j] = (live && (uint32_t)j < top_k) ? src2sorted[(size_t)row * top_k + j] : -1;
+    // amax, clamp and cast on packed bf16 bit patterns, as in the stand-alone quantizer's fast path
+    const uint32_t d0[4] = {raw0.x, raw0.y, raw0.z, raw0.w}, d1[4] = {raw1.x, raw1.y, raw1.z, raw1.w};
+    uint32_t a0[4], a1[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        a0[i] = d0[i] & 0x7FFF7FFFu;
+        a1[i] = d1[i] & 0x7FFF7FFFu;
+    }
+    uint32_t m = pk_max_u16(pk_max_u16(pk_max_u16(a0[0], a0[1]), pk_max_u16(a0[2], a0[3])),
+                            pk_max_u16(pk_max_u16(a1[0], a1[1]), pk_max_u16(a1[2], a1[3])));
+    m = pk_max_u16(m, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)m, 0xB1, 0xF, 0xF, true));      // the block's other lane
     const uint32_t amax = max(m & 0xFFFFu, m >> 16);
     const int e = block_exp_from_bf16_amax(amax, kEmaxE4M3);
-    if (!live) return;
     const uint32_t lim = (((uint32_t)(e + kEmaxE4M3 + 127) << 7) | 0x60u) * 0x10001u;
     const float scale = __uint_as_float((uint32_t)(e + 127) << 23);
-    uint32_t c[4];
+    uint32_t c0[4], c1[4];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) c[i] = pk_min_u16(a[i], lim) | (d[i] & 0x80008000u);
-    const uint32_t w0 = cvt_scaled_pk4<CMX_FMT_E4M3>(c[0], c[1], scale);
-    const uint32_t w1 = cvt_scaled_pk4<CMX_FMT_E4M3>(c[2], c[3], scale);
-    const uint8_t sbyte = (uint8_t)(e + 127);
+    for (int i = 0; i < 4; ++i) {
+        c0[i] = pk_min_u16(a0[i], lim) | (d0[i] & 0x80008000u);
+        c1[i] = pk_min_u16(a1[i], lim) | (d1[i] & 0x80008000u);
+    }
+    uint32_t w0 = cvt_scaled_pk4<CMX_FMT_E4M3>(c0[0], c0[1], scale), w1 = cvt_scaled_pk4<CMX_FMT_E4M3>(c0[2], c0[3], scale);
+    uint32_t w2 = cvt_scaled_pk4<CMX_FMT_E4M3>(c1[0], c1[1], scale), w3 = cvt_scaled_pk4<CMX_FMT_E4M3>(c1[2], c1[3], scale);
+    if (amax >= 0x7F80u) {                                  // Inf / NaN in the block (rare)
+        patch_nonfinite_fp8<CMX_FMT_E4M3, false>(d0, w0, w1);
+        patch_nonfinite_fp8<CMX_FMT_E4M3, false>(d1, w2, w3);
+    }
+    const uint32_t sbyte = (uint32_t)(e + 127) & 0xFFu;
+    // scale bytes of blocks b .. b+3 (lanes l, l+2, l+4, l+6 of one 16-lane row) in the lane of the first
+    uint32_t s4 = sbyte;
+    if constexpr (VEC_SCALES) {
+        s4 |= (uint32_t)__builtin_amdgcn_update_dpp(0, (int)sbyte, 0x102, 0xF, 0xF, true) << 8;     // row_shl:2
+        s4 |= (uint32_t)__builtin_amdgcn_update_dpp(0, (int)sbyte, 0x104, 0xF, 0xF, true) << 16;    // row_shl:4
+        s4 |= (uint32_t)__builtin_amdgcn_update_dpp(0, (int)sbyte, 0x106, 0xF, 0xF, true) << 24;    // row_shl:6
+    }
+    if (!live) return;
     const bool pad = (kb == nb - 1) && (nb & 1u);
-    for (uint32_t r = 0; r < top_k; ++r) {
-        const int32_t dst = src2sorted[(size_t)row * top_k + r];
-        if (dst < 0) continue;
-        *reinterpret_cast<uint2*>(out_codes + (size_t)dst * ld_out + col) = make_uint2(w0, w1);
-        if (q == 0) {
-            uint8_t* s = out_scales + (size_t)dst * ld_outs;
-            s[kb] = sbyte;
-            if (pad) s[nb] = 127;
+    const uint4 codes = make_uint4(w0, w1, w2, w3);
+    for (uint32_t r0 = 0; r0 < top_k; r0 += 8) {
+        if (r0 > 0) {
+#pragma unroll
+            for (int j = 0; j < 8; ++j) dst[j] = r0 + j < top_k ? src2sorted[(size_t)row * top_k + r0 + j] : -1;
+        }
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            if (dst[j] < 0) continue;
+            *reinterpret_cast<uint4*>(out_codes + (size_t)dst[j] * ld_out + col) = codes;
+            uint8_t* s = out_scales + (size_t)dst[j] * ld_outs;
+            if constexpr (VEC_SCALES) {
+                if ((threadIdx.x & 7u) == 0) *reinterpret_cast<uint32_t*>(s + kb) = s4;
+            } else if (h == 0) {
+                s[kb] = (uint8_t)sbyte;
+                if (pad) s[nb] = 127;
+            }
         }
     }
 }
 
 // ---- weighted top-k combine -----------------------------------------------------------------------
-// One workgroup per token; a lane owns 8 consecutive hidden elements per step.
+// Rows of whole 16-byte vectors: one lane per (token, 8 hidden elements), items numbered token-major, so that
+// every lane has the same amount of work whatever the hidden size.  A lane reads its token's eight row indices
+// and weights (the same addresses across most of a wavefront: one transaction), issues the eight 16-byte gathers
+// together and only then starts the arithmetic.
+__global__ __launch_bounds__(256) void unpermute_vec_kernel(const uint16_t* __restrict__ y, uint32_t ld_y, uint32_t rows,
+                                                             const int32_t* __restrict__ src2sorted,
+                                                             const float* __restrict__ probs, uint16_t* __restrict__ out,
+                                                             uint32_t ld_out, uint32_t nvec, uint32_t top_k,
+                                                             uint32_t total_items) {
+    const uint32_t item = blockIdx.x * 256 + threadIdx.x;
+    if (item >= total_items) return;
+    const uint32_t t = item / nvec, v = item - t * nvec;
+    const int32_t* idx = src2sorted + (size_t)t * top_k;
+    const float* wts = probs + (size_t)t * top_k;
+    float acc[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) acc[i] = 0.0f;
+    for (uint32_t k0 = 0; k0 < top_k; k0 += 8) {
+        int32_t r[8];
+        float w[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const bool in = k0 + j < top_k;
+            r[j] = in ? idx[k0 + j] : -1;
+            w[j] = in ? wts[k0 + j] : 0.0f;
+        }
+        uint4 raw[8];
+        bool ok[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            ok[j] = r[j] >= 0 && (uint32_t)r[j] < rows;
+            raw[j] = ok[j] ? *reinterpret_cast<const uint4*>(y + (size_t)r[j] * ld_y + v * 8) : make_uint4(0, 0, 0, 0);
+        }
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            if (k0 + j >= top_k) break;
+            const uint32_t dd[4] = {raw[j].x, raw[j].y, raw[j].z, raw[j].w};
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                // separate multiply and add (no fused multiply-add): Muls then Add in fp32, in k order; a row that is
+                // out of range contributes an exact zero
+                const float t0 = ok[j] ? __fmul_rn(__uint_as_float(dd[i] << 16), w[j]) : 0.0f;
+                const float t1 = ok[j] ? __fmul_rn(__uint_as_float(dd[i] & 0xFFFF0000u), w[j]) : 0.0f;
+                acc[2 * i] = (k0 + j) == 0 ? t0 : __fadd_rn(acc[2 * i], t0);
+                acc[2 * i + 1] = (k0 + j) == 0 ? t1 : __fadd_rn(acc[2 * i + 1], t1);
+            }
+        }
+    }
+    uint32_t o[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) o[i] = f32_to_bf16(acc[2 * i]) | (f32_to_bf16(acc[2 * i + 1]) << 16);
+    *reinterpret_cast<uint4*>(out + (size_t)t * ld_out + v * 8) = make_uint4(o[0], o[1], o[2], o[3]);
+}
+
+// Any hidden size (the ragged tail element by element): one workgroup per token; a lane owns 8 consecutive hidden
+// elements per step.
 template <int KMAX>
 __global__ __launch_bounds__(256) void unpermute_kernel(const uint16_t* __restrict__ y, uint32_t ld_y, uint32_t rows,
                                                          const int32_t* __restrict__ src2sorted,
@@ -348,15 +441,21 @@ extern "C" int cmx_quant_scatter(const void* x, uint32_t ld_x, const int32_t* sr
     if (tokens == 0 || k == 0 || top_k == 0) return CMX_OK;
     CMX_REQUIRE(k % 32 == 0, "k must be a multiple of 32");
     CMX_REQUIRE(ld_x >= k && ld_x % 8 == 0 && aligned16(x), "input rows must be 16-byte aligned");
-    CMX_REQUIRE(ld_out >= k && ld_out % 8 == 0 && (reinterpret_cast<uintptr_t>(out_codes) & 7u) == 0,
-                "output rows must be 8-byte aligned");
+    CMX_REQUIRE(ld_out >= k && ld_out % 16 == 0 && aligned16(out_codes), "output rows must be 16-byte aligned");
     CMX_REQUIRE(ld_outs >= scale_cols(k), "scale pitch too small");
     const uint32_t nb = k / 32;
     CMX_REQUIRE((uint64_t)tokens * nb < (1ull << 32), "too many blocks for one launch");
     const uint32_t total = tokens * nb;
-    hipLaunchKernelGGL(quant_scatter_kernel, dim3(ceil_div(total, 64)), dim3(256), 0, static_cast<hipStream_t>(stream),
-                       static_cast<const uint16_t*>(x), ld_x, src2sorted, out_codes, ld_out, out_scales, ld_outs, tokens,
-                       k, top_k, nb, total);
+    const bool vec_scales = nb % 4 == 0 && ld_outs % 4 == 0 && (reinterpret_cast<uintptr_t>(out_scales) & 3u) == 0;
+    const dim3 grid(ceil_div(total, 128));
+    const uint16_t* xp = static_cast<const uint16_t*>(x);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (vec_scales)
+        hipLaunchKernelGGL((quant_scatter_kernel<true>), grid, dim3(256), 0, s, xp, ld_x, src2sorted, out_codes, ld_out,
+                           out_scales, ld_outs, tokens, k, top_k, nb, total);
+    else
+        hipLaunchKernelGGL((quant_scatter_kernel<false>), grid, dim3(256), 0, s, xp, ld_x, src2sorted, out_codes, ld_out,
+                           out_scales, ld_outs, tokens, k, top_k, nb, total);
     CMX_LAUNCH_CHECK();
     return CMX_OK;
 }
@@ -368,6 +467,7 @@ extern "C" int cmx_int8_quant_scatter(const void* x, uint32_t ld_x, const int32_
     CMX_REQUIRE(x && codes && scales, "null pointer");
     if (tokens == 0 || k == 0) return CMX_OK;
     CMX_REQUIRE(top_k >= 1 && top_k <= 256, "top_k must be in [1, 256]");
+    CMX_REQUIRE((uint64_t)tokens * top_k < (1ull << 32), "tokens * top_k must stay below 2^32");
     CMX_REQUIRE(src2sorted != nullptr || top_k == 1, "without a destination table every token has one destination");
     CMX_REQUIRE(k % 8 == 0, "k must be a multiple of 8");
     CMX_REQUIRE(ld_x >= k && ld_x % 8 == 0 && aligned16(x), "input rows must be 16-byte aligned");
@@ -388,9 +488,16 @@ extern "C" int cmx_moe_token_unpermute(const void* y, uint32_t ld_y, uint32_t ro
     CMX_REQUIRE(top_k > 0 && top_k <= (uint32_t)kMaxTopK, "top_k must be in [1, 64]");
     CMX_REQUIRE(ld_y >= hidden && ld_out >= hidden, "row pitch smaller than a row");
     CMX_REQUIRE(ld_y % 8 == 0 && ld_out % 8 == 0 && aligned16(y) && aligned16(out), "rows must be 16-byte aligned");
-    hipLaunchKernelGGL((unpermute_kernel<kMaxTopK>), dim3(tokens), dim3(256), 0, static_cast<hipStream_t>(stream),
-                       static_cast<const uint16_t*>(y), ld_y, rows, src2sorted, probs, static_cast<uint16_t*>(out),
-                       ld_out, hidden, top_k);
+    if (hidden % 8 == 0 && (uint64_t)tokens * (hidden / 8) < (1ull << 32)) {
+        const uint32_t nvec = hidden / 8, total = tokens * nvec;
+        hipLaunchKernelGGL(unpermute_vec_kernel, dim3(ceil_div(total, 256)), dim3(256), 0, static_cast<hipStream_t>(stream),
+                           static_cast<const uint16_t*>(y), ld_y, rows, src2sorted, probs, static_cast<uint16_t*>(out),
+                           ld_out, nvec, top_k, total);
+    } else {
+        hipLaunchKernelGGL((unpermute_kernel<kMaxTopK>), dim3(tokens), dim3(256), 0, static_cast<hipStream_t>(stream),
+                           static_cast<const uint16_t*>(y), ld_y, rows, src2sorted, probs, static_cast<uint16_t*>(out),
+                           ld_out, hidden, top_k);
+    }
     CMX_LAUNCH_CHECK();
     return CMX_OK;
 }

@@ -180,6 +180,26 @@ __device__ __forceinline__ uint32_t cvt_scaled_pk4(uint32_t d0, uint32_t d1, flo
     return __builtin_bit_cast(uint32_t, o);
 }
 
+// Non-finite elements, which only a block whose maximum is Inf or NaN can hold (a rare branch behind the casts):
+// Inf becomes the largest magnitude code with its sign, NaN the NaN code with its sign under the nearest-even cast
+// and +0 under the table search -- what the reference's Python golden produces.  d = the block's eight bf16
+// bit patterns of this lane, w0 / w1 = their eight codes.
+template <int FMT, bool LUT>
+__device__ __forceinline__ void patch_nonfinite_fp8(const uint32_t (&d)[4], uint32_t& w0, uint32_t& w1) {
+    constexpr uint32_t maxc = FMT == CMX_FMT_E5M2 ? 0x7Bu : 0x7Eu;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+        const uint32_t pat = (j & 1) ? d[j >> 1] >> 16 : d[j >> 1] & 0xFFFFu;
+        const uint32_t mag = pat & 0x7FFFu;
+        if (mag >= 0x7F80u) {
+            const uint32_t sign = (pat >> 8) & 0x80u;
+            const uint32_t code = mag == 0x7F80u ? (maxc | sign) : (LUT ? 0u : (0x7Fu | sign));
+            const uint32_t sh = 8 * (j & 3);
+            uint32_t& w = j < 4 ? w0 : w1;
+            w = (w & ~(0xFFu << sh)) | (code << sh);
+        }
+    }
+}
 
 typedef float v2f32 __attribute__((ext_vector_type(2)));
 // two floats -> packed bf16 (a in the low half), round-to-nearest-even in hardware

@@ -22,6 +22,7 @@
 // weight panels in its own L2.
 #include <atomic>
 #include <type_traits>
+#include <vector>
 
 #include "mx_common.h"
 
@@ -954,16 +955,39 @@ int current_device_slot(int* dev_out) {
     return CMX_OK;
 }
 
-template <typename K>
-int allow_dynamic_lds(K kfn, size_t bytes, PerDeviceFlag& flag) {
+// Every kernel that needs more dynamic LDS than the default limit is listed here at load time (one entry per
+// instantiation that a launch function names), so that cmx_init can raise all the limits up front and no first
+// call has to -- hipFuncSetAttribute is not allowed while a stream is being captured into a graph.
+struct LdsKernel {
+    const void* fn;
+    int bytes;
+    PerDeviceFlag* flag;
+};
+std::vector<LdsKernel>& lds_registry() {
+    static std::vector<LdsKernel> v;
+    return v;
+}
+template <auto KFN, size_t SMEM>
+struct LdsSetup {
+    static inline PerDeviceFlag flag{};
+    static inline const bool registered = (lds_registry().push_back({reinterpret_cast<const void*>(KFN), (int)SMEM, &flag}), true);
+};
+
+int allow_dynamic_lds(const void* kfn, int bytes, PerDeviceFlag& flag) {
     int dev = 0;
     int rc = current_device_slot(&dev);
     if (rc != CMX_OK) return rc;
     if (!flag.done[dev].load(std::memory_order_acquire)) {
-        CMX_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kfn), hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes));
+        CMX_HIP(hipFuncSetAttribute(kfn, hipFuncAttributeMaxDynamicSharedMemorySize, bytes));
         flag.done[dev].store(true, std::memory_order_release);
     }
     return CMX_OK;
+}
+// raises the limit of KFN on the current device unless cmx_init or an earlier call has done so
+template <auto KFN, size_t SMEM>
+int allow_dynamic_lds() {
+    (void)LdsSetup<KFN, SMEM>::registered;
+    return allow_dynamic_lds(reinterpret_cast<const void*>(KFN), (int)SMEM, LdsSetup<KFN, SMEM>::flag);
 }
 
 int cu_count(int* out) {
@@ -985,9 +1009,8 @@ template <int FMT, int TW, int TM, int WW, int WM, int EPI, bool FAST>
 int launch_gemm_impl(const GemmParams& p, uint32_t max_m_tiles, hipStream_t s) {
     constexpr int kScaleDw = FMT == CMX_FMT_E2M1 ? 2 : 1;
     constexpr size_t smem = 2 * ((TW + TM) * kSlabBytes + (TW + TM) * 4 * kScaleDw);
-    auto kfn = mx_gemm_kernel<FMT, TW, TM, WW, WM, EPI, FAST>;
-    static PerDeviceFlag lds_allowed;
-    if (int rc = allow_dynamic_lds(kfn, smem, lds_allowed); rc != CMX_OK) return rc;
+    constexpr auto kfn = mx_gemm_kernel<FMT, TW, TM, WW, WM, EPI, FAST>;
+    if (int rc = allow_dynamic_lds<kfn, smem>(); rc != CMX_OK) return rc;
     const uint64_t tiles = (uint64_t)max_m_tiles * p.w_tiles;
     CMX_REQUIRE(tiles > 0 && tiles < (1ull << 31), "tile count out of range");
     hipLaunchKernelGGL(kfn, dim3((uint32_t)tiles), dim3(64 * WW * WM), smem, s, p);
@@ -999,9 +1022,8 @@ template <int FMT, int TW, int TM, int WW, int WM, int EPI>
 int launch_gemm_dl(const GemmParams& p, uint32_t max_m_tiles, hipStream_t s) {
     constexpr int kScaleDw = FMT == CMX_FMT_E2M1 ? 2 : 1;
     constexpr size_t smem = 2 * (TW + TM) * kSlabBytes + 2 * (TW + TM) * kScaleDw * 4;
-    auto kfn = mx_gemm_dl_kernel<FMT, TW, TM, WW, WM, EPI>;
-    static PerDeviceFlag lds_allowed;
-    if (int rc = allow_dynamic_lds(kfn, smem, lds_allowed); rc != CMX_OK) return rc;
+    constexpr auto kfn = mx_gemm_dl_kernel<FMT, TW, TM, WW, WM, EPI>;
+    if (int rc = allow_dynamic_lds<kfn, smem>(); rc != CMX_OK) return rc;
     const uint64_t tiles = (uint64_t)max_m_tiles * p.w_tiles;
     CMX_REQUIRE(tiles > 0 && tiles < (1ull << 31), "tile count out of range");
     hipLaunchKernelGGL(kfn, dim3((uint32_t)tiles), dim3(64 * WW * WM), smem, s, p);
@@ -1013,9 +1035,8 @@ template <int FMT, int EPI, int TM, int WW, int WM, int NSLOT>
 int launch_gemm_pipe(const GemmParams& p, uint32_t max_m_tiles, hipStream_t s) {
     // tile ring, scale ring (two-slot kernels: two blocks of 16 bytes per row), next-tile mailbox
     constexpr size_t smem = NSLOT * (256 + TM) * kSlabBytes + (NSLOT == 2 ? 2 * (256 + TM) * 16 : NSLOT * (256 + TM) * 4) + 16;
-    auto kfn = mx_gemm_pipe_kernel<FMT, EPI, TM, WW, WM, NSLOT>;
-    static PerDeviceFlag lds_allowed;
-    if (int rc = allow_dynamic_lds(kfn, smem, lds_allowed); rc != CMX_OK) return rc;
+    constexpr auto kfn = mx_gemm_pipe_kernel<FMT, EPI, TM, WW, WM, NSLOT>;
+    if (int rc = allow_dynamic_lds<kfn, smem>(); rc != CMX_OK) return rc;
     const uint64_t tiles = (uint64_t)max_m_tiles * p.w_tiles;
     CMX_REQUIRE(tiles > 0 && tiles < (1ull << 31), "tile count out of range");
     uint32_t grid = (uint32_t)tiles;
@@ -1034,9 +1055,8 @@ int launch_gemm_pipe(const GemmParams& p, uint32_t max_m_tiles, hipStream_t s) {
 template <int EPI, int WW, int WM>
 int launch_gemm_pipe_fp4(const GemmParams& p, uint32_t max_m_tiles, hipStream_t s) {
     constexpr size_t smem = 2 * 512 * kSlabBytes + 2 * 512 * 16 + 16;     // tile ring, ring of two scale blocks, next-tile mailbox
-    auto kfn = mx_gemm_pipe_fp4_kernel<EPI, WW, WM>;
-    static PerDeviceFlag lds_allowed;
-    if (int rc = allow_dynamic_lds(kfn, smem, lds_allowed); rc != CMX_OK) return rc;
+    constexpr auto kfn = mx_gemm_pipe_fp4_kernel<EPI, WW, WM>;
+    if (int rc = allow_dynamic_lds<kfn, smem>(); rc != CMX_OK) return rc;
     const uint64_t tiles = (uint64_t)max_m_tiles * p.w_tiles;
     CMX_REQUIRE(tiles > 0 && tiles < (1ull << 31), "tile count out of range");
     uint32_t grid = (uint32_t)tiles;
@@ -1052,7 +1072,13 @@ int launch_gemm_pipe_fp4(const GemmParams& p, uint32_t max_m_tiles, hipStream_t 
     return CMX_OK;
 }
 
-bool g_disable_dl = false;   // tuning/test hook: force the register-staged kernels
+// The test build of this file (CMX_TEST_HOOKS, linked into the test library only) can force the register-staged
+// kernels and pin the tile shape, so that tests reach every compiled instantiation; the product has neither switch.
+#ifdef CMX_TEST_HOOKS
+bool g_disable_dl = false;
+#else
+constexpr bool g_disable_dl = false;
+#endif
 
 template <int FMT, int TW, int TM, int WW, int WM, int EPI>
 int launch_gemm(const GemmParams& p, uint32_t max_m_tiles, hipStream_t s) {
@@ -1070,7 +1096,11 @@ struct TileChoice {
     int tw, tm, waves;
 };
 
-TileChoice g_force_tile = {0, 0, 0};   // test/tuning hook: tw == 0 -> heuristic
+#ifdef CMX_TEST_HOOKS
+TileChoice g_force_tile = {0, 0, 0};   // tw == 0 -> heuristic
+#else
+constexpr TileChoice g_force_tile = {0, 0, 0};
+#endif
 
 // waves: at 256 x 256 "4" and "5" select the hand-scheduled kernel in its 2 x 2 and 4 x 1 wavefront layouts
 // when the problem is eligible for it (8-bit elements, whole 512-byte K blocks).  2 x 2 reads a fifth less
@@ -1173,16 +1203,18 @@ bool scales_dword_aligned(const void* as, uint32_t ld_as, const void* ws, uint32
 
 }  // namespace cmx
 
+#ifdef CMX_TEST_HOOKS
 extern "C" int cmx_debug_disable_streaming(int off) {
     cmx::g_disable_dl = off != 0;
     return CMX_OK;
 }
 
-// tuning/test hook: pin the tile shape and wavefront count (tw = 0 restores the heuristic)
+// pin the tile shape and wavefront count of every later matmul call (tw = 0 restores the heuristic)
 extern "C" int cmx_debug_force_tile(int tw, int tm, int waves) {
     cmx::g_force_tile = (tw > 0 && tm > 0) ? cmx::TileChoice{tw, tm, waves > 0 ? waves : 4} : cmx::TileChoice{0, 0, 0};
     return CMX_OK;
 }
+#endif
 
 extern "C" int cmx_mx_gemm(const uint8_t* a, uint32_t lda, const uint8_t* a_scale, uint32_t ld_as, const uint8_t* b,
                            uint32_t ldb, const uint8_t* b_scale, uint32_t ld_bs, void* c, uint32_t ldc, uint32_t m,
@@ -1259,16 +1291,19 @@ extern "C" int cmx_mx_gmm(const uint8_t* a, uint32_t lda, const uint8_t* a_scale
     using namespace cmx;
     if (m_total == 0 || n == 0) return CMX_OK;
     const uint32_t kbytes = fmt == CMX_FMT_E2M1 ? k / 2 : k;
-    int rc = check_operands(a, lda, a_scale, ld_as, b, kbytes, b_scale, k / 32, k, fmt);
+    // weight scale rows are as every producer writes them: padded to an even count (the quantizer, the
+    // reference generator's transposed even-padded matrix, the host operators' ScaleCols(k))
+    const uint32_t ld_ws = scale_cols(k);
+    int rc = check_operands(a, lda, a_scale, ld_as, b, kbytes, b_scale, ld_ws, k, fmt);
     if (rc != CMX_OK) return rc;
     CMX_REQUIRE(c && ldc >= n, "bad output");
     CMX_REQUIRE(out_type == CMX_OUT_BF16 || out_type == CMX_OUT_FP16 || out_type == CMX_OUT_FP32, "unknown output type");
     GemmParams p{};
     p.a = a; p.a_scale = a_scale; p.w = b; p.w_scale = b_scale; p.c = c;
-    p.lda = lda; p.ld_as = ld_as; p.ldw = kbytes; p.ld_ws = k / 32; p.ldc = ldc;
+    p.lda = lda; p.ld_as = ld_as; p.ldw = kbytes; p.ld_ws = ld_ws; p.ldc = ldc;
     p.m = m_total; p.n = n; p.kbytes = kbytes; p.kblocks = k / 32; p.out_type = out_type;
-    p.scale_vec = scales_dword_aligned(a_scale, ld_as, b_scale, k / 32);
-    p.scale_vec16 = scales_aligned16(a_scale, ld_as, b_scale, k / 32);
+    p.scale_vec = scales_dword_aligned(a_scale, ld_as, b_scale, ld_ws);
+    p.scale_vec16 = scales_aligned16(a_scale, ld_as, b_scale, ld_ws);
     return gmm_common(p, group_sizes, groups, m_total, workspace, fmt, false, static_cast<hipStream_t>(stream));
 }
 
@@ -1330,14 +1365,14 @@ extern "C" int cmx_int8_gmm_dequant_swiglu(const int8_t* a, uint32_t lda, const 
     return launch_gemm_dl<kFmtI8, kTile, kTile, 2, 4, kEpiI8DequantSwiglu>(p, m_total / kTile + groups, s);
 }
 
-extern "C" int cmx_mx_gmm_swiglu_quant(const uint8_t* a, uint32_t lda, const uint8_t* a_scale, uint32_t ld_as,
-                                       const uint8_t* b, const uint8_t* b_scale, uint8_t* act_codes, uint32_t ld_act,
-                                       uint8_t* act_scales, uint32_t ld_acts, void* act_bf16,
-                                       const int32_t* group_sizes, uint32_t groups, uint32_t m_total, uint32_t n,
-                                       uint32_t k, void* workspace, cmx_stream_t stream) {
-    using namespace cmx;
-    if (m_total == 0 || n == 0) return CMX_OK;
-    int rc = check_operands(a, lda, a_scale, ld_as, b, k, b_scale, k / 32, k, CMX_FMT_E4M3);
+namespace cmx {
+namespace {
+int gmm_swiglu_quant(const uint8_t* a, uint32_t lda, const uint8_t* a_scale, uint32_t ld_as, const uint8_t* b,
+                     const uint8_t* b_scale, uint8_t* act_codes, uint32_t ld_act, uint8_t* act_scales, uint32_t ld_acts,
+                     void* act_bf16, const int32_t* group_sizes, uint32_t groups, uint32_t m_total, uint32_t n, uint32_t k,
+                     void* workspace, cmx_stream_t stream) {
+    const uint32_t ld_ws = scale_cols(k);      // even-padded weight scale rows, as in cmx_mx_gmm
+    int rc = check_operands(a, lda, a_scale, ld_as, b, k, b_scale, ld_ws, k, CMX_FMT_E4M3);
     if (rc != CMX_OK) return rc;
     CMX_REQUIRE(n % 64 == 0, "n must be a multiple of 64 (gate|up halves of whole MX blocks)");
     CMX_REQUIRE(act_codes && act_scales, "null pointer");
@@ -1348,9 +1383,33 @@ extern "C" int cmx_mx_gmm_swiglu_quant(const uint8_t* a, uint32_t lda, const uin
     p.a = a; p.a_scale = a_scale; p.w = b; p.w_scale = b_scale;
     p.act_codes = act_codes; p.act_scales = act_scales; p.act_bf16 = static_cast<uint16_t*>(act_bf16);
     p.ld_act = ld_act; p.ld_acts = ld_acts;
-    p.lda = lda; p.ld_as = ld_as; p.ldw = k; p.ld_ws = k / 32;
+    p.lda = lda; p.ld_as = ld_as; p.ldw = k; p.ld_ws = ld_ws;
     p.m = m_total; p.n = n; p.kbytes = k; p.kblocks = k / 32; p.out_type = CMX_OUT_BF16;
-    p.scale_vec = scales_dword_aligned(a_scale, ld_as, b_scale, k / 32);
-    p.scale_vec16 = scales_aligned16(a_scale, ld_as, b_scale, k / 32);
+    p.scale_vec = scales_dword_aligned(a_scale, ld_as, b_scale, ld_ws);
+    p.scale_vec16 = scales_aligned16(a_scale, ld_as, b_scale, ld_ws);
     return gmm_common(p, group_sizes, groups, m_total, workspace, CMX_FMT_E4M3, true, static_cast<hipStream_t>(stream));
+}
+
+}  // namespace
+}  // namespace cmx
+
+extern "C" int cmx_mx_gmm_swiglu_quant(const uint8_t* a, uint32_t lda, const uint8_t* a_scale, uint32_t ld_as,
+                                       const uint8_t* b, const uint8_t* b_scale, uint8_t* act_codes, uint32_t ld_act,
+                                       uint8_t* act_scales, uint32_t ld_acts, void* act_bf16,
+                                       const int32_t* group_sizes, uint32_t groups, uint32_t m_total, uint32_t n,
+                                       uint32_t k, void* workspace, cmx_stream_t stream) {
+    if (m_total == 0 || n == 0) return CMX_OK;
+    return cmx::gmm_swiglu_quant(a, lda, a_scale, ld_as, b, b_scale, act_codes, ld_act, act_scales, ld_acts, act_bf16,
+                                 group_sizes, groups, m_total, n, k, workspace, stream);
+}
+
+// One-time set-up on the current device: raises the dynamic-LDS limit of every matmul kernel and reads the CU count,
+// so that no later call has to (not allowed inside a stream capture).  Optional: every entry point still does what
+// it needs on first use.
+extern "C" int cmx_init(void) {
+    using namespace cmx;
+    for (const LdsKernel& k : lds_registry())
+        if (int rc = allow_dynamic_lds(k.fn, k.bytes, *k.flag); rc != CMX_OK) return rc;
+    int cus = 0;
+    return cu_count(&cus);
 }

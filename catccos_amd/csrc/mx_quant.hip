@@ -75,7 +75,11 @@ __global__ __launch_bounds__(kThreads) void mx_quant_kernel(const uint16_t* __re
             amax = amax > hi ? amax : hi;
         }
         amax = quad_max(amax);
-        const int e = block_exp_from_bf16_amax(amax, emax);
+        int e = block_exp_from_bf16_amax(amax, emax);
+        // a block whose maximum is Inf or NaN: the 8-bit formats take the exponent field as it is (255), the 4-bit
+        // formats the largest exponent for Inf and a NaN scale (byte 255, every code 0) for NaN
+        const bool nonfinite = amax >= 0x7F80u;
+        if (kFp4 && nonfinite) e = 127;
 
         float y[8];
 #pragma unroll
@@ -91,6 +95,7 @@ __global__ __launch_bounds__(kThreads) void mx_quant_kernel(const uint16_t* __re
             uint32_t pk = 0;
 #pragma unroll
             for (int i = 0; i < 8; ++i) pk |= fp4_encode<FMT>(y[i], LUT) << (4 * i);
+            if (amax > 0x7F80u) pk = 0;
             uint8_t* o = codes + (size_t)row * ld_codes + (col >> 1);
             if (vec_out) {
                 if (col < cols) *reinterpret_cast<uint32_t*>(o) = pk;
@@ -122,6 +127,7 @@ __global__ __launch_bounds__(kThreads) void mx_quant_kernel(const uint16_t* __re
                 w0 = f0;
                 w1 = f1;
             }
+            if (nonfinite) patch_nonfinite_fp8<FMT, LUT>(d, w0, w1);
             uint8_t* o = codes + (size_t)row * ld_codes + col;
             if (vec_out) {
                 if (col < cols) *reinterpret_cast<uint2*>(o) = make_uint2(w0, w1);
@@ -135,8 +141,8 @@ __global__ __launch_bounds__(kThreads) void mx_quant_kernel(const uint16_t* __re
         }
         if (q == 0) {
             uint8_t* s = scales + (size_t)row * ld_scales;
-            s[kb] = (uint8_t)(e + 127);
-            if (kb == nb - 1 && (nb & 1u)) s[nb] = 127;   // pad the scale row to an even count with 1.0
+            s[kb] = (kFp4 && amax > 0x7F80u) ? (uint8_t)255 : (uint8_t)(e + 127);
+            if (kb == nb - 1 && (nb & 1u) && ld_scales > nb) s[nb] = 127;   // pad the scale row to an even count with 1.0
         }
     }
 }
@@ -190,8 +196,9 @@ __global__ __launch_bounds__(kThreads) void mx_quant_rne8_kernel(const uint8_t* 
         uint32_t c[4];
 #pragma unroll
         for (int i = 0; i < 4; ++i) c[i] = pk_min_u16(a[i], lim) | (d[i] & 0x80008000u);
-        const uint32_t w0 = cvt_scaled_pk4<FMT>(c[0], c[1], scale);
-        const uint32_t w1 = cvt_scaled_pk4<FMT>(c[2], c[3], scale);
+        uint32_t w0 = cvt_scaled_pk4<FMT>(c[0], c[1], scale);
+        uint32_t w1 = cvt_scaled_pk4<FMT>(c[2], c[3], scale);
+        if (amax >= 0x7F80u) patch_nonfinite_fp8<FMT, false>(d, w0, w1);      // Inf / NaN in the block (rare)
         if (row < rows) *reinterpret_cast<uint2*>(codes + (size_t)row * ld_codes + out_off) = make_uint2(w0, w1);
         my_e = (int)q == u ? e : my_e;
     }
@@ -199,7 +206,7 @@ __global__ __launch_bounds__(kThreads) void mx_quant_rne8_kernel(const uint8_t* 
     if (srow < rows) {
         uint8_t* sp = scales + (size_t)srow * ld_scales;
         sp[kb] = (uint8_t)(my_e + 127);
-        if (kb == nb - 1 && (nb & 1u)) sp[nb] = 127;       // pad the scale row to an even count with 1.0
+        if (kb == nb - 1 && (nb & 1u) && ld_scales > nb) sp[nb] = 127;       // pad the scale row to an even count with 1.0
     }
 }
 
@@ -259,7 +266,9 @@ extern "C" int cmx_mx_quant(const void* x, uint32_t ld_x, uint8_t* codes, uint32
     const uint32_t nb = ceil_div(cols, 32);
     const bool fp4 = fmt == CMX_FMT_E2M1 || fmt == CMX_FMT_E1M2;
     const uint32_t code_cols = fp4 ? ceil_div(cols, 2) : cols;
-    CMX_REQUIRE(ld_x >= cols && ld_codes >= code_cols && ld_scales >= scale_cols(cols), "row pitch smaller than row");
+    // a scale pitch of exactly ceil(cols / 32) columns selects the unpadded scale rows of the reference's
+    // mx_quant_allgather files; any larger pitch must hold the even-padded row
+    CMX_REQUIRE(ld_x >= cols && ld_codes >= code_cols && (ld_scales == nb || ld_scales >= scale_cols(cols)), "row pitch smaller than row");
     CMX_REQUIRE((uint64_t)rows * nb < (1ull << 32), "too many blocks for one launch");
     const uint32_t total = rows * nb;
     const int vec_in = (cols % 8 == 0) && (ld_x % 8 == 0) && aligned16(x);

@@ -64,17 +64,14 @@ public:
         return blockBytes < static_cast<size_t>(perRank);
     }
 
-    // Launch: scales need an even count per row in the library; the file format has exactly n/32.
+    // Launch: the file format has exactly n/32 scale bytes per row; a scale pitch of exactly that many columns
+    // makes the library write unpadded scale rows (odd block counts such as n = 96 included).
     static int Launch(void* stream, const KernelParams& params, const CocTilingParams& t, uint32_t rankId)
     {
         const uint32_t scaleCols = t.n / MX_BLOCK_SIZE;
         const uint32_t codeCols = t.n / PackRatio();
         uint8_t* codes = params.ptrC + static_cast<size_t>(rankId) * t.m * codeCols;
         uint8_t* scales = params.ptrB + static_cast<size_t>(rankId) * t.m * scaleCols;
-        if (scaleCols % 2 != 0) {
-            cmx_rt_stream_sync(stream);
-            return CMX_EINVAL;      // an odd block count would need a padded scale row
-        }
         return cmx_mx_quant(params.ptrA, t.n, codes, codeCols, scales, scaleCols, t.m, t.n, ElementFormat(), RoundMode(),
                             stream);
     }

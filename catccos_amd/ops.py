@@ -199,6 +199,11 @@ def mx_gmm_swiglu_quant(a, a_scale, b, b_scale, group_sizes, k: int, want_bf16: 
     return codes, scales, act
 
 
+def init() -> None:
+    """cmx_init on the current device."""
+    _lib.check(_lib.load().cmx_init())
+
+
 def moe_init_routing(expert_idx: torch.Tensor, experts: int):
     """expert_idx int32 [T, topK] -> (sorted2src, src2sorted, counts) int32."""
     _need_cuda(expert_idx)
@@ -277,11 +282,4 @@ def dispatch_ffn_combine(x, expert_idx, gate_weight, w1, w1_scale, w2, w2_scale,
     _lib.check(lib.catccos_ascend950_dispatch_ffn_combine(
         0, _stream(), 0, _p(x), _p(expert_idx), _p(gate_weight), _p(w1), _p(w1_scale), _p(w2), _p(w2_scale), _p(out),
         _p(workspace), None, m, k, n, e, top_k, 1))
-    return out
-
-
-def mfma_raw_probe(a_regs, b_regs, sa, sb, fmt: str, opsel: int, shape: int) -> torch.Tensor:
-    out = torch.zeros((64, 16 if shape == 0 else 4), dtype=torch.float32, device=a_regs.device)
-    _lib.check(_lib.load().cmx_mfma_raw_probe(_p(a_regs), _p(b_regs), _p(sa), _p(sb), _p(out), FMT[fmt], opsel, shape,
-                                              _stream()))
     return out

@@ -81,6 +81,7 @@ def _ffn(x, expert_idx, gate_weight, w1, w1_scale, w2, w2_scale):
     _check(k % 256 == 0 and n % 512 == 0, "K must be divisible by 256 and N by 512")
     _check(0 < local_experts <= (2 ** 31 - 1) // rank_size, "total expert count exceeds the int32 kernel limit")
     _check(0 < top_k <= local_experts * rank_size, "invalid TopK")
+    _check(top_k <= 64, "TopK exceeds the weighted combine's limit of 64")
     _check(m <= (2 ** 31 - 1) // rank_size // top_k, "routed row count exceeds the int32 kernel limit")
     k2, scale_k, scale_k2 = n // 2, k // 32, n // 64
     _check(expert_idx.shape[0] == m and gate_weight.shape == expert_idx.shape, "expected [M, TopK] routing")

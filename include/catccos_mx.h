@@ -45,6 +45,11 @@ typedef void* cmx_stream_t;
 int cmx_version(void);
 const char* cmx_last_error(void);
 
+/* One-time set-up on the current device (no counterpart in the reference, whose kernels need none): raises the
+ * dynamic-LDS limit of every matmul kernel and reads the CU count.  Optional -- every entry point does what it needs on first use -- but a caller
+ * that captures streams into graphs must call it first: raising a kernel's LDS limit is not allowed during capture. */
+int cmx_init(void);
+
 /* ------------------------------------------------------------------------------------------
  * Runtime shim: what the host plugin layer needs from the device runtime.
  * Replaces aclrtMalloc / aclrtFree / aclrtMallocHost / aclrtFreeHost / aclrtMemcpy /
@@ -74,7 +79,16 @@ int cmx_rt_stream_sync(cmx_stream_t stream);
  *
  *   x       bf16 [rows, cols], row pitch ld_x elements
  *   codes   u8   [rows, cols] (FP4: [rows, ceil(cols/2)]), row pitch ld_codes bytes
- *   scales  u8   [rows, RoundUp2(ceil(cols/32))], row pitch ld_scales bytes; padding column = 127
+ *   scales  u8   [rows, RoundUp2(ceil(cols/32))], row pitch ld_scales bytes; padding column = 127.
+ *           A pitch of exactly ceil(cols/32) selects unpadded scale rows (the [M, N/32] file of
+ *           examples/ascend950_mx_quant_allgather/mx_quant_allgather_host.h:47-87): no padding column is written.
+ *
+ * Non-finite input follows the golden, not the reference device (which writes scale 0xFF and NaN codes for such
+ * a block, comm_block_mx_quant.hpp:496-515).  A block whose maximum is Inf or NaN: 8-bit formats take the
+ * exponent field as it is (scale byte 247 for E4M3, 240 for E5M2) and scale the finite elements by it, +-Inf
+ * becomes the largest code with its sign, NaN the NaN code 0x7F | sign (CMX_ROUND_RNE) or code 0
+ * (CMX_ROUND_LUT).  4-bit formats: an Inf maximum gives scale byte 254 and +-Inf the largest code; a NaN
+ * maximum gives scale byte 255 and code 0 for every element of the block.
  * ---------------------------------------------------------------------------------------- */
 int cmx_mx_quant(const void* x, uint32_t ld_x, uint8_t* codes, uint32_t ld_codes, uint8_t* scales,
                  uint32_t ld_scales, uint32_t rows, uint32_t cols, int fmt, int round_mode, cmx_stream_t stream);
@@ -108,7 +122,8 @@ int cmx_mx_gemm(const uint8_t* a, uint32_t lda, const uint8_t* a_scale, uint32_t
  *
  *   group_sizes  int32 [groups] ON DEVICE (rows per expert, in order; zeros allowed)
  *   a / a_scale  rows of all groups back to back, m_total = sum(group_sizes) rows
- *   b / b_scale  [groups, n, k] / [groups, n, k/32], dense
+ *   b / b_scale  [groups, n, k] / [groups, n, RoundUp2(k/32)], dense (scale rows padded to an even count, as the
+ *                quantizer and the reference's generators write them; no padding when k is a multiple of 64)
  *   c            [m_total, n]
  *   workspace    >= cmx_mx_gmm_workspace_bytes(groups) bytes (tile schedule metadata)
  * Rows beyond sum(group_sizes) (up to m_total) are left untouched.
@@ -237,7 +252,7 @@ int cmx_moe_init_routing(const int32_t* expert_idx, uint32_t tokens, uint32_t to
  *
  *   x           bf16 [tokens, k]
  *   src2sorted  int32 [tokens*top_k]; negative destinations are skipped
- *   out_codes   row r at out_codes + r*ld_out;  out_scales row r at out_scales + r*ld_outs
+ *   out_codes   row r at out_codes + r*ld_out (16-byte aligned rows);  out_scales row r at out_scales + r*ld_outs
  * The reference's packed wire row [codes k | scales RoundUp2(k/32) | pad to 32 B] is the case
  * out_scales = out_codes + k, ld_out = ld_outs = cmx_packed_row_bytes(k).
  * ---------------------------------------------------------------------------------------- */
@@ -268,6 +283,7 @@ int cmx_moe_token_unpermute(const void* y, uint32_t ld_y, uint32_t rows, const i
  *   w1 E4M3 [E,n,k], w1Scale [E,n,k/32]; w2 [E,k,n/2], w2Scale [E,k,n/64]; out bf16 [m,k]
  *   workspace >= catccos_ascend950_dispatch_ffn_combine_workspace_bytes(...) ; contents may be
  *   garbage on entry.
+ * topK <= min(localExperts, 64), m * topK < 2^31; every shape limit is checked before the first launch.
  * ---------------------------------------------------------------------------------------- */
 uint64_t catccos_ascend950_symmetric_bytes(void);
 size_t catccos_ascend950_dispatch_ffn_combine_workspace_bytes(uint32_t m, uint32_t k, uint32_t n,
@@ -287,24 +303,6 @@ typedef struct cmx_ffn_workspace_layout {
 } cmx_ffn_workspace_layout;
 int cmx_ffn_workspace_layout_get(uint32_t m, uint32_t k, uint32_t n, uint32_t localExperts, uint32_t topK,
                                  cmx_ffn_workspace_layout* layout);
-
-/* ------------------------------------------------------------------------------------------
- * Test and tuning hooks (no counterpart in the reference).
- *
- * cmx_mfma_raw_probe: one wavefront executes one block-scaled MFMA on caller-supplied registers, so
- * the operand/scale/accumulator lane layout the GEMM kernels rely on can be pinned by known-answer
- * tests.  a_regs/b_regs: int32 [64 lanes][8]; sa/sb: int32 [64] (scale VGPR per lane, byte `opsel`
- * is used for both operands); out: fp32 [64][16] (shape 0: 32x32x64) or [64][4] (shape 1: 16x16x128).
- *
- * cmx_debug_force_tile: (tw, tm, waves) overrides the tile heuristic of every later matmul call in
- * this process so tests can cover every compiled tile shape; tw <= 0 restores the heuristic.
- * cmx_debug_disable_streaming: non-zero forces the register-staged kernels instead of the
- * LDS-streaming ones.  Neither hook is thread safe; both return CMX_OK.
- * ---------------------------------------------------------------------------------------- */
-int cmx_mfma_raw_probe(const void* a_regs, const void* b_regs, const int32_t* sa, const int32_t* sb, float* out,
-                       int fmt, int opsel, int shape, cmx_stream_t stream);
-int cmx_debug_force_tile(int tw, int tm, int waves);
-int cmx_debug_disable_streaming(int off);
 
 #ifdef __cplusplus
 }

@@ -89,14 +89,31 @@ int mxo_quant_bf16(const uint16_t* x, int rows, int cols, int fmt, int mode, uin
         for (int b = 0; b < nb; ++b) {
             const int lo = b * 32, hi = lo + 32 < cols ? lo + 32 : cols;
             float amax = 0.0f;
+            int has_nan = 0;
             for (int c = lo; c < hi; ++c) {
                 float a = fabsf(bf16_to_f32(x[(size_t)r * cols + c]));
+                if (a != a) has_nan = 1;
                 if (a > amax) amax = a;
             }
-            const int e = block_exp(amax, emaxs[fmt]);
-            scales[(size_t)r * sc + b] = (uint8_t)(e + 127);
+            /* A maximum of Inf or NaN, as the golden treats it (torch's amax returns NaN if the block holds one):
+             * the 8-bit path reads the exponent field, 255, of either (:181-189); the 4-bit path takes
+             * floor(log2(.)) in floating point (:429-432): Inf -> the largest exponent, NaN -> a NaN scale
+             * (byte 255) that makes every quotient NaN and every code 0. */
+            int e = block_exp(amax, emaxs[fmt]);
+            if (fmt != 2 && (has_nan || isinf(amax))) e = 128 - emaxs[fmt];
+            if (fmt == 2 && isinf(amax)) e = 127;
+            const int nan_scale = fmt == 2 && has_nan;
+            scales[(size_t)r * sc + b] = nan_scale ? 255 : (uint8_t)(e + 127);
             for (int c = lo; c < hi; ++c) {
                 const float xv = bf16_to_f32(x[(size_t)r * cols + c]);
+                if (nan_scale) {
+                    codes[(size_t)r * cols + c] = 0;
+                    continue;
+                }
+                if (xv != xv) {         /* NaN element: NaN code with its sign under the cast, +0 under the table search */
+                    codes[(size_t)r * cols + c] = (fmt != 2 && mode == 0) ? (uint8_t)(0x7F | (signbit_of(xv) ? 0x80 : 0)) : 0;
+                    continue;
+                }
                 double y = ldexp((double)xv, -e);
                 if (y > maxv[fmt]) y = maxv[fmt];
                 if (y < -maxv[fmt]) y = -maxv[fmt];

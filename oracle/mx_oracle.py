@@ -13,12 +13,17 @@ reference checkout).  Bit-level conventions:
 * "RNE" = IEEE round-to-nearest-even; "LUT" = nearest table value with ties to
   the smaller magnitude and -0 canonicalised to +0 (first-index arg-min).
 
-Pinning status (see tests/test_oracle_*.py): E8M0 exponent, E4M3/E5M2 RNE (vs the
-torch CPU cast and brute force over all bf16 patterns), E4M3/E2M1 LUT (vs the
-256-/16-entry arg-min definition), FP4 packing, bf16 RNE, routing, combine,
-workspace sizing are pinned.  MX GEMM results are pinned only through tolerance
-and special cases (the bit-level accumulate order of the reference's matmul
-lives in an absent third-party library): exact GEMM bits are "parity unpinned".
+Pinning status (see tests/test_oracle_*.py, tests/test_golden_fixtures.py): E8M0 exponent,
+E4M3/E5M2 RNE (vs the torch CPU cast and brute force over all bf16 patterns), E4M3/E2M1
+LUT (vs the 256-/16-entry arg-min definition), FP4 packing, bf16 RNE, routing, combine,
+workspace sizing (literal hand-computed sums) and both acceptance rules (literal cases at
+and one step beyond every threshold) are pinned.  The quantizers (every format and
+rounding, ties, signed zeros, tiny / all-zero blocks, Inf and NaN) and the whole FFN chain
+are also pinned bit for bit by vectors that the reference's own Python goldens produced
+(tests/golden/*.npz, made by tests/golden/make_fixtures.py).  MX GEMM results of the
+reference DEVICE are pinned only through tolerance and special cases (the bit-level
+accumulate order of its matmul lives in an absent third-party library): exact device GEMM
+bits are "parity unpinned".
 """
 from __future__ import annotations
 
@@ -172,7 +177,7 @@ def _fp8_rne(y, man_bits: int, bias: int, max_code: int) -> np.ndarray:
     code_n = (rounded >> drop) - ((127 - bias) << man_bits)
     # subnormals: value = k * 2^(1-bias-man_bits), k = RNE(|y| / step)
     step_log2 = 1 - bias - man_bits
-    mag = np.abs(y).astype(np.float64)
+    mag = np.where(np.isnan(y), 0.0, np.abs(y).astype(np.float64))       # NaN is patched in below
     code_s = np.rint(mag * 2.0 ** (-step_log2)).astype(np.int64)
     min_normal = 2.0 ** (1 - bias)
     code = np.where(mag < min_normal, code_s, code_n)
@@ -208,7 +213,11 @@ def _lut_pos_encode(y, pos: np.ndarray) -> np.ndarray:
 
 
 def fp8_encode_lut(y, fmt: str = "E4M3") -> np.ndarray:
-    idx, neg = _lut_pos_encode(y, _FP8[fmt][:128])
+    """Table-search encode.  A NaN element comes out as code 0: the golden's torch.searchsorted puts NaN at
+    index 0, whose table value 0 is then canonicalised to +0 (pinned by the reference-made vectors)."""
+    y = np.ascontiguousarray(y, dtype=np.float32)
+    nan = np.isnan(y)
+    idx, neg = _lut_pos_encode(np.where(nan, np.float32(0), y), _FP8[fmt][:128])
     return (idx | np.where(neg, 0x80, 0).astype(np.uint8)).astype(np.uint8)
 
 
@@ -256,7 +265,8 @@ def fp4_encode_rne(y, fmt: str = "E2M1") -> np.ndarray:
         mid = (float(tab[i]) + float(tab[i + 1])) / 2
         up = (mag > mid) | ((mag == mid) & (((i + 1) & 1) == 0))
         code = np.where(up, i + 1, code)
-    return (code | np.where(np.signbit(y), 8, 0)).astype(np.uint8)
+    # a NaN (only reachable in a block whose maximum is NaN) encodes as +0, like the table search
+    return np.where(np.isnan(y), 0, code | np.where(np.signbit(y), 8, 0)).astype(np.uint8)
 
 
 def pack_fp4(codes) -> np.ndarray:
@@ -315,12 +325,22 @@ def mx_quant(x, fmt: str = "E4M3", mode: str | None = None):
     else:
         xp = x
     blocks = xp.reshape(m, nb, BLOCK)
-    amax = np.abs(blocks).max(axis=-1)
+    with np.errstate(invalid="ignore"):
+        amax = np.abs(blocks).max(axis=-1)                  # NaN if the block holds one
     exp = e8m0_exp(amax, f["emax"])
+    nan_block = np.zeros(amax.shape, dtype=bool)
+    if fmt not in _FP8:
+        # the FP4 golden takes floor(log2(amax)) in floating point (:429-432): an Inf maximum gives the largest
+        # exponent, a NaN maximum a NaN scale (byte 255) and with it NaN quotients, which the table search
+        # sends to code 0
+        exp = np.where(np.isinf(amax), 127, exp).astype(np.int32)
+        nan_block = np.isnan(amax)
     # division by an exact power of two == scaling by 2^-exp (ldexp is exact)
-    scaled = np.ldexp(blocks, -exp[..., None]).astype(np.float32)
+    with np.errstate(invalid="ignore", over="ignore"):
+        scaled = np.ldexp(blocks, -exp[..., None]).astype(np.float32)
     mv = np.float32(f["max_value"])
-    scaled = np.clip(scaled, -mv, mv)
+    scaled = np.clip(scaled, -mv, mv)                       # NaN stays NaN, as torch.clamp leaves it
+    scaled = np.where(nan_block[..., None], np.float32(np.nan), scaled)
     if fmt == "E4M3":
         codes = e4m3_encode_rne(scaled) if mode == "rne" else fp8_encode_lut(scaled, "E4M3")
     elif fmt == "E5M2":
@@ -329,7 +349,7 @@ def mx_quant(x, fmt: str = "E4M3", mode: str | None = None):
         codes = fp4_encode_rne(scaled, fmt) if mode == "rne" else fp4_encode_lut(scaled, fmt)
     codes = codes.reshape(m, pn)[:, :n]
     sc = np.full((m, scale_cols(n)), E8M0_BIAS, dtype=np.uint8)
-    sc[:, :nb] = e8m0_byte(exp)
+    sc[:, :nb] = np.where(nan_block, np.uint8(255), e8m0_byte(exp))
     return np.ascontiguousarray(codes), sc
 
 
@@ -401,11 +421,6 @@ def to_file_layout_fp4(codes, scales, trans: bool):
     if not trans:
         return pack_fp4(codes), np.ascontiguousarray(pairs)
     return pack_fp4(np.ascontiguousarray(codes.T)), np.ascontiguousarray(pairs.transpose(1, 0, 2))
-
-
-def mx_gemm_bf16(*args, **kw) -> np.ndarray:
-    """bf16 result (bit pattern) of :func:`mx_gemm_f32` (gen_data_moe.py:650)."""
-    return f32_to_bf16_bits(mx_gemm_f32(*args, **kw))
 
 
 def group_offsets(counts) -> np.ndarray:
@@ -485,11 +500,6 @@ def moe_init_routing(expert_idx, expert_num: int):
     return sorted2src, src2sorted, counts
 
 
-def permute_rows(x, sorted2src, top_k: int):
-    """permuted[i] = x[sorted2src[i] // topK]   (gen_data_moe.py:54-55)"""
-    return np.asarray(x)[np.asarray(sorted2src, dtype=np.int64) // top_k]
-
-
 def packed_row_bytes(k: int) -> int:
     """[codes K | scales RoundUp2(K/32) | pad to 32 B]
     (comm_block_mx_quant.hpp:326-330)."""
@@ -566,8 +576,9 @@ def moe_ffn(x_bits, expert_idx, probs, w1_codes, w1_scales, w2_codes, w2_scales,
 
 def unpermute_cpu_bf16(y_bits, sorted2src, probs) -> np.ndarray:
     """The golden's CPU fallback combine (gen_data_moe.py:60-70): bf16 multiply,
-    bf16 ``index_add_`` in sorted-row order.  Kept to show the build's fp32
-    combine stays inside the acceptance tolerance of this variant."""
+    bf16 ``index_add_`` in sorted-row order.  This is what the reference-made FFN vector
+    (tests/golden/ffn_tiny.npz) was combined with; the product follows the device's fp32
+    combine (:func:`unpermute_combine`) and stays inside the acceptance tolerance of this variant."""
     y = bf16_bits_to_f32(y_bits)
     probs = np.asarray(probs, dtype=np.float32)
     t, top_k = probs.shape
@@ -603,6 +614,33 @@ def verify_bf16(out_bits, golden_f32, k: int):
     err = int(np.count_nonzero(np.abs(diff) - rtol * tmax > 0))
     eb = float(abs(np.mean(diff / tmax)))
     return (err == 0 and eb <= 2.0 ** -7), err, eb
+
+
+def verify_double_golden_bf16(out_bits, golden_f32, golden_low_bits):
+    """The double-golden acceptance of the dense MXFP8 matmul (verify_result.py:117-134, 244-306 with
+    OpTypes.COMPUTE_FLOAT_HIGH_PRECISION and a bf16 output, as
+    ascend950_mxfp8_matmul_reduce_scatter/scripts/run.sh:57-62 calls it): the output's maximum and mean relative
+    error and its RMSE against the fp32 golden, each divided by max(the same figure of the bf16 "low" golden,
+    2^-8), must stay below 10, 2 and 2, and |mean((out - gold) / max(1, |gold|))| <= 2^-7; non-finite positions
+    must coincide.  Returns (ok, max_ratio, mean_ratio, rmse_ratio, eb)."""
+    out = bf16_bits_to_f32(out_bits).astype(np.float32).ravel()
+    gold = np.asarray(golden_f32, dtype=np.float32).ravel()
+    low = bf16_bits_to_f32(golden_low_bits).astype(np.float32).ravel()
+    if np.count_nonzero(np.isfinite(out) != np.isfinite(gold)):
+        return False, float("inf"), float("inf"), float("inf"), 0.0
+    out = np.where(np.isfinite(out), out, np.float32(0))
+    gold = np.where(np.isfinite(gold), gold, np.float32(0))
+    low = np.where(np.isfinite(low), low, np.float32(0))
+    thr = np.float32(2.0 ** -8)
+    eps = np.float32(1e-7)
+    d_out, d_low = out - gold, low - gold
+    eb = float(abs(np.mean(d_out / np.maximum(np.float32(1), np.abs(gold)))))
+    rel_out, rel_low = np.abs(d_out) / (np.abs(gold) + eps), np.abs(d_low) / (np.abs(gold) + eps)
+    rmse_out, rmse_low = np.sqrt(np.mean(d_out ** 2)), np.sqrt(np.mean(d_low ** 2))
+    r_max = float(rel_out.max() / max(rel_low.max(), thr))
+    r_mean = float(rel_out.mean() / max(rel_low.mean(), thr))
+    r_rmse = float(rmse_out / max(rmse_low, thr))
+    return (r_max < 10 and r_mean < 2 and r_rmse < 2 and eb <= 2.0 ** -7), r_max, r_mean, r_rmse, eb
 
 
 # --------------------------------------------------------------------------- #

@@ -18,7 +18,7 @@ For every instantiation that the library dispatches to, this script compiles tha
 (device only, nothing is linked or run) and reports the spills and waits found between the first and the last
 MFMA.  Run it after any change to the kernels, the epilogues or their helpers:
 
-    python3 catccos_amd/csrc/check_pipe_schedule.py          # a few seconds per kernel
+    python3 tests/check_pipe_schedule.py          # a few seconds per kernel
 
 Exit status 0 when every kernel is clean.
 """
@@ -30,8 +30,8 @@ import subprocess
 import sys
 import tempfile
 
-HERE = os.path.dirname(os.path.abspath(__file__))
-ROOT = os.path.dirname(os.path.dirname(HERE))
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HERE = os.path.join(ROOT, "catccos_amd", "csrc")          # where the kernel sources live
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
          f"-I{os.path.join(ROOT, 'include')}", f"-I{HERE}", "-S", "--cuda-device-only", "-Wno-unused-command-line-argument"]

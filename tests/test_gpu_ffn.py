@@ -65,6 +65,41 @@ def test_ffn_vs_oracle(tokens, k, n, experts, top_k):
     assert torch.equal(out, out2)
 
 
+def test_several_shapes_on_one_dirty_workspace():
+    """The reference's case-list mode runs several shapes in one process on one workspace that was poisoned once
+    (examples/ascend950_dispatch_ffn_combine/main.cpp:150-170, 217-252): a large shape first, then smaller ones on
+    what it left behind, then the large one again.  Every result must equal that of a run on a fresh workspace."""
+    from catccos_amd import ops
+    shapes = [(512, 512, 1024, 32, 4), (4, 256, 512, 4, 2), (300, 256, 512, 8, 8), (64, 512, 1024, 16, 6), (512, 512, 1024, 32, 4)]
+    big = max(ops.ffn_workspace_bytes(*s) for s in shapes)
+    shared = torch.full((big,), 0xA5, dtype=torch.uint8, device="cuda")
+    for i, (tokens, k, n, experts, top_k) in enumerate(shapes):
+        x, idx, p, w1q, w1s, w2q, w2s = _make(tokens, k, n, experts, top_k, seed=tokens + 11)
+        args = (bf16_dev(x), dev(idx), dev(p), dev(w1q), dev(w1s), dev(w2q), dev(w2s))
+        fresh = torch.zeros(ops.ffn_workspace_bytes(tokens, k, n, experts, top_k), dtype=torch.uint8, device="cuda")
+        want = ops.dispatch_ffn_combine(*args, workspace=fresh)
+        got = ops.dispatch_ffn_combine(*args, workspace=shared)
+        assert torch.equal(got.view(torch.int16), want.view(torch.int16)), (i, tokens)
+        if tokens <= 64:                                    # and against the oracle chain
+            gold = O.bf16_bits_to_f32(O.moe_ffn(x, idx, p, w1q, w1s, w2q, w2s))
+            bad, worst = close_bf16(host(got), gold)
+            assert bad <= got.numel() // 1000 and worst <= 5e-2, (bad, worst)
+
+
+def test_ffn_rejects_top_k_beyond_the_combine_limit_before_any_launch():
+    from catccos_amd import _lib
+    lib = _lib.load()
+    z = torch.zeros(1 << 20, dtype=torch.uint8, device="cuda")
+    out = torch.full((1 << 16,), 0x5A, dtype=torch.uint8, device="cuda")
+    ws = torch.full((1 << 22,), 0xA5, dtype=torch.uint8, device="cuda")
+    p = z.data_ptr()
+    rc = lib.catccos_ascend950_dispatch_ffn_combine(0, None, 0, p, p, p, p, p, p, p, out.data_ptr(), ws.data_ptr(), None,
+                                                    2, 256, 512, 128, 65, 1)
+    torch.cuda.synchronize()
+    assert rc == -1 and b"64" in lib.cmx_last_error()
+    assert bool((ws == 0xA5).all()) and bool((out == 0x5A).all())          # nothing was launched
+
+
 def test_workspace_size_matches_reference_formula():
     from catccos_amd import ops
     for (m, k, n, e, t) in [(4, 7168, 4096, 16, 6), (512, 7168, 4096, 16, 6), (8192, 7168, 4096, 256, 8), (256, 7168, 1024, 16, 6)]:

@@ -5,16 +5,16 @@ import torch
 
 from oracle import mx_oracle as O
 from catccos_amd import workloads as W
-from tests.gpu_util import dev, host, close_bf16
+from tests.gpu_util import dev, host, close_bf16, hooked_library, hooks_lib
 
 pytestmark = pytest.mark.gpu
 
 
 @pytest.fixture(autouse=True)
-def _reset_tile():
-    yield
-    from catccos_amd import _lib
-    _lib.load().cmx_debug_force_tile(0, 0, 0)
+def _hooked():
+    """These tests pin tile shapes: they run the package's front end on the test build of the library."""
+    with hooked_library():
+        yield
 
 
 def _weights(rng, g, n, k, std=0.05, fmt="E4M3"):
@@ -27,7 +27,7 @@ def _weights(rng, g, n, k, std=0.05, fmt="E4M3"):
 def test_gmm_fp8_ragged_groups(tile, counts):
     from catccos_amd import ops, _lib
     if tile:
-        _lib.load().cmx_debug_force_tile(*tile)
+        hooks_lib().cmx_debug_force_tile(*tile)
     rng = np.random.default_rng(sum(counts))
     n, k = 320, 256
     m = sum(counts)
@@ -49,7 +49,7 @@ def test_gmm_many_ragged_groups_every_row(tile):
     exactly once with its own group's weights."""
     from catccos_amd import ops, _lib
     if tile:
-        _lib.load().cmx_debug_force_tile(*tile)
+        hooks_lib().cmx_debug_force_tile(*tile)
     rng = np.random.default_rng(77)
     counts = [int(c) for c in rng.integers(0, 700, size=36)] + [256, 512, 0, 128, 128, 1, 255]
     n, k = 256, 512
@@ -78,7 +78,7 @@ def test_more_tiles_than_workgroups_every_row(fmt, k, waves):
     tile: the load stream crosses the tile boundary, the next tile comes from the per-XCD counters, and every
     row of every group must still come out right, with the rows past the groups untouched."""
     from catccos_amd import ops, _lib
-    _lib.load().cmx_debug_force_tile(256, 256, waves)
+    hooks_lib().cmx_debug_force_tile(256, 256, waves)
     rng = np.random.default_rng(91)
     counts = [int(c) for c in rng.integers(0, 700, size=36)] + [256, 512, 0, 128, 1, 255]
     n = 1024
@@ -105,7 +105,7 @@ def test_swiglu_requant_more_tiles_than_workgroups(waves):
     """The fused GMM1 epilogue on about 300 tiles: the persistent kernels (2 x 2 and 4 x 1 wavefronts) go through
     the epilogue and on to a next tile."""
     from catccos_amd import ops, _lib
-    _lib.load().cmx_debug_force_tile(256, 256, waves)
+    hooks_lib().cmx_debug_force_tile(256, 256, waves)
     rng = np.random.default_rng(92)
     counts = [int(c) for c in rng.integers(0, 700, size=36)] + [256, 512, 0, 128, 1, 255]
     n, k = 1024, 512
@@ -129,7 +129,7 @@ def test_group_sizes_that_overrun_the_buffers_are_cut_off(tile):
     sizes count as zero, so the kernels never leave the caller's buffers."""
     from catccos_amd import ops, _lib
     if tile:
-        _lib.load().cmx_debug_force_tile(*tile)
+        hooks_lib().cmx_debug_force_tile(*tile)
     rng = np.random.default_rng(41)
     n, k, m = 192, 512, 400
     aq, asc = O.mx_quant(O.bf16_round(rng.standard_normal((m, k)).astype(np.float32)))
@@ -185,7 +185,7 @@ def test_swiglu_requant_with_groups_about_one_tile_long():
 def test_gmm_fp4_ragged_groups(tile, k):
     from catccos_amd import ops, _lib
     if tile:
-        _lib.load().cmx_debug_force_tile(*tile)
+        hooks_lib().cmx_debug_force_tile(*tile)
     rng = np.random.default_rng(3)
     counts = [40, 0, 129, 300]
     n = 256
@@ -207,7 +207,7 @@ def test_gmm1_swiglu_requant(tile):
     bit-exact against the oracle quantizer applied to the kernel's own bf16 SwiGLU output."""
     from catccos_amd import ops, _lib
     if tile:
-        _lib.load().cmx_debug_force_tile(*tile)
+        hooks_lib().cmx_debug_force_tile(*tile)
     rng = np.random.default_rng(12)
     counts = [70, 0, 300, 3, 130]
     n, k = 512, 512
@@ -253,3 +253,35 @@ def test_config3_routing_shape_small_hidden():
     assert bad == 0, (bad, worst)
     wq2, ws2 = O.mx_quant_bf16(host(act), "E4M3", "rne")
     assert np.array_equal(host(scales), ws2) and np.array_equal(host(codes), wq2)
+
+
+@pytest.mark.parametrize("k", [96, 160, 32])
+@pytest.mark.parametrize("fmt", ["E4M3", "E2M1"])
+def test_gmm_odd_block_count_weight_scales_have_the_even_padded_pitch(k, fmt):
+    """K / 32 odd: scale rows, of the weights too, are padded to an even count (what the quantizer and the reference's
+    generators write), so every weight row after the first sits at a pitch of K/32 + 1 bytes."""
+    from catccos_amd import ops
+    rng = np.random.default_rng(k)
+    counts = [3, 0, 70, 129]
+    n, m = 192, sum(counts)
+    mode = "lut" if fmt == "E2M1" else "rne"
+    a, a_s = ops.mx_quant(dev(O.f32_to_bf16_bits(rng.standard_normal((m, k)).astype(np.float32))).view(torch.bfloat16), fmt, mode)
+    wq, ws = [], []
+    for _ in counts:                                        # weights straight from the library's own quantizer
+        q, s = ops.mx_quant(dev(O.f32_to_bf16_bits(rng.standard_normal((n, k)).astype(np.float32))).view(torch.bfloat16), fmt, "lut")
+        wq.append(q)
+        ws.append(s)
+    w, w_s = torch.stack(wq).contiguous(), torch.stack(ws).contiguous()
+    assert w_s.shape[2] == O.scale_cols(k) == k // 32 + 1
+    c = ops.mx_gmm(a, a_s, w, w_s, dev(np.array(counts, dtype=np.int32)), k, fmt)
+    un = (lambda t: O.unpack_fp4(host(t))) if fmt == "E2M1" else host
+    gold = O.mx_gmm_f32(un(a), host(a_s), np.stack([un(q) for q in wq]), host(w_s), counts, fmt, fmt)
+    bad, worst = close_bf16(host(c), gold, atol=5e-2 if fmt == "E2M1" else 1e-2)
+    assert bad == 0, (bad, worst)
+    if fmt == "E4M3" and n % 64 == 0:
+        codes, scales, act = ops.mx_gmm_swiglu_quant(a, a_s, w, w_s, dev(np.array(counts, dtype=np.int32)), k, want_bf16=True)
+        q2, s2 = O.mx_quant_bf16(host(act), "E4M3", "rne")
+        assert np.array_equal(host(codes), q2) and np.array_equal(host(scales), s2)
+        _, act_g, _, _ = O.gmm1_swiglu_quant(host(a), host(a_s), host(w), host(w_s), counts)
+        bad, worst = close_bf16(host(act), O.bf16_bits_to_f32(act_g), rtol=2e-2)
+        assert bad == 0, (bad, worst)

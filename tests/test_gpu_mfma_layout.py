@@ -9,7 +9,7 @@ import pytest
 import torch
 
 from oracle import mx_oracle as O
-from tests.gpu_util import dev, host
+from tests.gpu_util import dev, host, mfma_raw_probe
 
 pytestmark = pytest.mark.gpu
 
@@ -54,7 +54,7 @@ def test_mfma_32x32x64_fp8_layout(opsel):
     a, as_ = O.mx_quant(rng.standard_normal((32, 64)).astype(np.float32) * 0.2)
     ws, as_ = ws[:, :2], as_[:, :2]
     ws[5, 1] += 3; as_[7, 0] -= 2          # make the two K blocks of a row scale differently
-    out = ops.mfma_raw_probe(dev(_regs_fp8(w)), dev(_regs_fp8(a)), dev(_scale_regs(ws, opsel)),
+    out = mfma_raw_probe(dev(_regs_fp8(w)), dev(_regs_fp8(a)), dev(_scale_regs(ws, opsel)),
                              dev(_scale_regs(as_, opsel)), "E4M3", opsel, 0)
     got = _unpack_acc(host(out))
     want = O.mx_dequant(w, ws).astype(np.float64) @ O.mx_dequant(a, as_).astype(np.float64).T
@@ -68,7 +68,7 @@ def test_mfma_32x32x64_fp4_layout():
     rng = np.random.default_rng(7)
     w, ws = O.mx_quant(rng.uniform(-2, 2, (32, 64)).astype(np.float32), "E2M1")
     a, as_ = O.mx_quant(rng.uniform(-2, 2, (32, 64)).astype(np.float32), "E2M1")
-    out = ops.mfma_raw_probe(dev(_regs_fp4(O.pack_fp4(w))), dev(_regs_fp4(O.pack_fp4(a))), dev(_scale_regs(ws[:, :2], 1)),
+    out = mfma_raw_probe(dev(_regs_fp4(O.pack_fp4(w))), dev(_regs_fp4(O.pack_fp4(a))), dev(_scale_regs(ws[:, :2], 1)),
                              dev(_scale_regs(as_[:, :2], 1)), "E2M1", 1, 0)
     got = _unpack_acc(host(out))
     want = O.mx_dequant(w, ws, "E2M1").astype(np.float64) @ O.mx_dequant(a, as_, "E2M1").astype(np.float64).T
@@ -83,7 +83,7 @@ def test_mfma_one_hot_locates_every_operand_byte():
     for (i, k) in [(0, 0), (3, 31), (17, 32), (31, 63), (9, 40)]:
         w = np.zeros((32, 64), dtype=np.uint8)
         w[i, k] = 0x40      # 2.0
-        out = ops.mfma_raw_probe(dev(_regs_fp8(w)), dev(_regs_fp8(ones)), dev(_scale_regs(unit, 0)),
+        out = mfma_raw_probe(dev(_regs_fp8(w)), dev(_regs_fp8(ones)), dev(_scale_regs(unit, 0)),
                                  dev(_scale_regs(unit, 0)), "E4M3", 0, 0)
         got = _unpack_acc(host(out))
         want = np.zeros((32, 32), dtype=np.float32)

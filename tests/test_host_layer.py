@@ -79,6 +79,19 @@ def test_driver_quant(host_bin, tmp_path, fmt, ofmt):
 
 
 @pytest.mark.gpu
+def test_driver_quant_odd_block_count_writes_unpadded_scale_rows(host_bin, tmp_path):
+    """N = 96: the reference operator writes exactly N / 32 = 3 scale bytes per row (mx_quant_allgather_host.h:47-87)."""
+    rows, cols = 40, 96
+    x = W.activations_with_outliers(rows, cols, seed=6)
+    _write(tmp_path / "rank_0_input.bin", x)
+    r = _run(host_bin, "MxQuantAllGather", rows, 1, cols, "--data", tmp_path, "--fmt", "e4m3", "--poison")
+    assert r.returncode == 0, r.stdout + r.stderr
+    codes, scales = O.mx_quant_bf16(x, "E4M3", "rne")
+    assert np.array_equal(np.fromfile(tmp_path / "rank_0_output.bin", dtype=np.uint8).reshape(rows, cols), codes)
+    assert np.array_equal(np.fromfile(tmp_path / "rank_0_mxscale.bin", dtype=np.uint8).reshape(rows, 3), scales[:, :3])
+
+
+@pytest.mark.gpu
 def test_driver_mxfp8_matmul(host_bin, tmp_path):
     m, k, n = 192, 1024, 384
     rng = np.random.default_rng(11)

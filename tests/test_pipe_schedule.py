@@ -9,7 +9,7 @@ import shutil
 import pytest
 
 HERE = os.path.dirname(os.path.abspath(__file__))
-SCRIPT = os.path.join(os.path.dirname(HERE), "catccos_amd", "csrc", "check_pipe_schedule.py")
+SCRIPT = os.path.join(HERE, "check_pipe_schedule.py")
 spec = importlib.util.spec_from_file_location("check_pipe_schedule", SCRIPT)
 chk = importlib.util.module_from_spec(spec)
 spec.loader.exec_module(chk)
