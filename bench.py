@@ -184,7 +184,15 @@ def main() -> int:
         extra["copycal"] = {"bytes_read": nbytes, "bytes_written": nbytes, "avg_launch_us": tcopy * 1e6,
                             "GBs": 2 * nbytes / tcopy / 1e9}
         log(f"[copy calibration] 1 GiB -> 1 GiB in {tcopy*1e6:.1f} us = {2*nbytes/tcopy/1e9:.0f} GB/s")
-        del src, dst
+        # what the memory system gives a write-only and a read-only stream of the same size (torch's fill and
+        # reduction kernels): the practical ceilings next to which the write-heavy scatter and the read-heavy
+        # combine are to be read
+        tfill = hip_time(lambda: dst.zero_(), steps=5, warm=1)
+        src32 = src.view(torch.int32)
+        tread = hip_time(lambda: torch.max(src32), steps=5, warm=1)
+        extra["copycal"].update({"write_only_GBs": nbytes / tfill / 1e9, "read_only_GBs": nbytes / tread / 1e9})
+        log(f"[ceilings] write-only {nbytes/tfill/1e9:.0f} GB/s, read-only {nbytes/tread/1e9:.0f} GB/s")
+        del src, dst, src32
 
     if "quant" in want:
         M1, K1 = 4096, 7168

@@ -70,6 +70,9 @@ SIGNATURES = {
                                                      u32, u32, u32, u32, u32, i32]),
     "cmx_ffn_workspace_layout_get": (i32, [u32, u32, u32, u32, u32, C.POINTER(FfnWorkspaceLayout)]),
     "cmx_init": (i32, []),
+    "cmx_mx_gmm_noalloc_max_groups": (u32, []),
+    "cmx_mx_gmm_swiglu_quant_noalloc": (i32, [u8p, u32, u8p, u32, u8p, u8p, u8p, u32, u8p, u32, vp, i32p, u32, u32, u32,
+                                              u32, vp]),
 }
 
 _lib = None

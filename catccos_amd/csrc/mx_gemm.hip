@@ -1390,6 +1390,28 @@ int gmm_swiglu_quant(const uint8_t* a, uint32_t lda, const uint8_t* a_scale, uin
     return gmm_common(p, group_sizes, groups, m_total, workspace, CMX_FMT_E4M3, true, static_cast<hipStream_t>(stream));
 }
 
+// Schedule metadata of the allocation-free entry point (row offsets, m-tile prefix, per-XCD tile counters of up to
+// kStaticGroups groups): a fixed array in device memory instead of a caller's workspace.  Every device that runs
+// the library holds its own copy; its address on a device comes from hipGetSymbolAddress with that device current
+// (the array's name is only a host-side handle).
+constexpr uint32_t kStaticGroups = 4096;
+constexpr size_t kStaticScratchBytes = (2 * ((size_t)kStaticGroups + 1) + 8) * sizeof(int32_t);
+static __device__ __align__(256) unsigned char scratch[(kStaticScratchBytes + 255) / 256 * 256];
+
+int static_scratch(void** out) {
+    static std::atomic<void*> ptrs[kMaxDevices];
+    int dev = 0;
+    int rc = current_device_slot(&dev);
+    if (rc != CMX_OK) return rc;
+    void* q = ptrs[dev].load(std::memory_order_acquire);
+    if (q == nullptr) {
+        CMX_HIP(hipGetSymbolAddress(&q, HIP_SYMBOL(scratch)));
+        CMX_REQUIRE(q != nullptr, "no device address for the static scratch array");
+        ptrs[dev].store(q, std::memory_order_release);
+    }
+    *out = q;
+    return CMX_OK;
+}
 }  // namespace
 }  // namespace cmx
 
@@ -1403,13 +1425,33 @@ extern "C" int cmx_mx_gmm_swiglu_quant(const uint8_t* a, uint32_t lda, const uin
                                  group_sizes, groups, m_total, n, k, workspace, stream);
 }
 
-// One-time set-up on the current device: raises the dynamic-LDS limit of every matmul kernel and reads the CU count,
-// so that no later call has to (not allowed inside a stream capture).  Optional: every entry point still does what
-// it needs on first use.
+extern "C" uint32_t cmx_mx_gmm_noalloc_max_groups(void) { return cmx::kStaticGroups; }
+
+extern "C" int cmx_mx_gmm_swiglu_quant_noalloc(const uint8_t* a, uint32_t lda, const uint8_t* a_scale, uint32_t ld_as,
+                                               const uint8_t* b, const uint8_t* b_scale, uint8_t* act_codes,
+                                               uint32_t ld_act, uint8_t* act_scales, uint32_t ld_acts, void* act_bf16,
+                                               const int32_t* group_sizes, uint32_t groups, uint32_t m_total,
+                                               uint32_t n, uint32_t k, cmx_stream_t stream) {
+    using namespace cmx;
+    if (m_total == 0 || n == 0) return CMX_OK;
+    CMX_REQUIRE(groups <= kStaticGroups, "at most 4096 groups fit the static schedule array: use cmx_mx_gmm_swiglu_quant with a workspace");
+    void* meta = nullptr;
+    if (int rc = static_scratch(&meta); rc != CMX_OK) return rc;
+    // gmm_prepare_kernel rewrites every word of the metadata that the matmul kernel reads (and zeroes the tile
+    // counters), so nothing of an earlier call survives into this one
+    return gmm_swiglu_quant(a, lda, a_scale, ld_as, b, b_scale, act_codes, ld_act, act_scales, ld_acts, act_bf16,
+                            group_sizes, groups, m_total, n, k, meta, stream);
+}
+
+// One-time set-up on the current device: raises the dynamic-LDS limit of every matmul kernel, reads the CU count and
+// resolves the static schedule array, so that no later call has to (none of this is allowed, or wise, inside a
+// stream capture).  Optional: every entry point still does what it needs on first use.
 extern "C" int cmx_init(void) {
     using namespace cmx;
     for (const LdsKernel& k : lds_registry())
         if (int rc = allow_dynamic_lds(k.fn, k.bytes, *k.flag); rc != CMX_OK) return rc;
     int cus = 0;
-    return cu_count(&cus);
+    if (int rc = cu_count(&cus); rc != CMX_OK) return rc;
+    void* meta = nullptr;
+    return static_scratch(&meta);
 }

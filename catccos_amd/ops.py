@@ -199,6 +199,18 @@ def mx_gmm_swiglu_quant(a, a_scale, b, b_scale, group_sizes, k: int, want_bf16: 
     return codes, scales, act
 
 
+def mx_gmm_swiglu_quant_noalloc(a, a_scale, b, b_scale, group_sizes, k: int, codes, scales, act=None) -> None:
+    """cmx_mx_gmm_swiglu_quant_noalloc: the caller brings every buffer (codes [m, n/2], scales, optional bf16 act);
+    neither this wrapper nor the library allocates anything."""
+    _need_cuda(a, a_scale, b, b_scale, group_sizes, codes, scales)
+    assert b.is_contiguous() and b_scale.is_contiguous() and group_sizes.dtype == torch.int32
+    m, (g, n) = a.shape[0], b.shape[:2]
+    lib = _lib.load()
+    _lib.check(lib.cmx_mx_gmm_swiglu_quant_noalloc(_p(a), a.stride(0), _p(a_scale), a_scale.stride(0), _p(b), _p(b_scale),
+                                                   _p(codes), codes.stride(0), _p(scales), scales.stride(0), _p(act),
+                                                   _p(group_sizes), g, m, n, k, _stream()))
+
+
 def init() -> None:
     """cmx_init on the current device."""
     _lib.check(_lib.load().cmx_init())

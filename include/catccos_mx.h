@@ -46,7 +46,8 @@ int cmx_version(void);
 const char* cmx_last_error(void);
 
 /* One-time set-up on the current device (no counterpart in the reference, whose kernels need none): raises the
- * dynamic-LDS limit of every matmul kernel and reads the CU count.  Optional -- every entry point does what it needs on first use -- but a caller
+ * dynamic-LDS limit of every matmul kernel, reads the CU count and resolves the static schedule array of
+ * cmx_mx_gmm_swiglu_quant_noalloc.  Optional -- every entry point does what it needs on first use -- but a caller
  * that captures streams into graphs must call it first: raising a kernel's LDS limit is not allowed during capture. */
 int cmx_init(void);
 
@@ -154,6 +155,20 @@ int cmx_mx_gmm_swiglu_quant(const uint8_t* a, uint32_t lda, const uint8_t* a_sca
                             uint8_t* act_scales, uint32_t ld_acts, void* act_bf16, const int32_t* group_sizes,
                             uint32_t groups, uint32_t m_total, uint32_t n, uint32_t k, void* workspace,
                             cmx_stream_t stream);
+
+/* cmx_mx_gmm_swiglu_quant without a workspace argument and without any allocation: no counterpart in the
+ * reference; it is for callers that cannot allocate device memory (code under HIP graph capture, tight serving
+ * loops, harnesses that forbid it).  The tile schedule metadata lives in a fixed array inside the library's device
+ * image (33 KiB per device, held until the process ends), which admits at most cmx_mx_gmm_noalloc_max_groups()
+ * = 4096 groups; more are rejected with CMX_EINVAL.  All calls on one device share that array: calls that overlap
+ * on one device (different streams) race on it; calls on one stream do not.  Same results as
+ * cmx_mx_gmm_swiglu_quant.  Under stream capture call cmx_init() beforehand. */
+uint32_t cmx_mx_gmm_noalloc_max_groups(void);
+int cmx_mx_gmm_swiglu_quant_noalloc(const uint8_t* a, uint32_t lda, const uint8_t* a_scale, uint32_t ld_as,
+                                    const uint8_t* b, const uint8_t* b_scale, uint8_t* act_codes, uint32_t ld_act,
+                                    uint8_t* act_scales, uint32_t ld_acts, void* act_bf16,
+                                    const int32_t* group_sizes, uint32_t groups, uint32_t m_total, uint32_t n,
+                                    uint32_t k, cmx_stream_t stream);
 
 /* ------------------------------------------------------------------------------------------
  * Operands stored with K as the slow axis.
