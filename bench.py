@@ -285,10 +285,12 @@ def main() -> int:
             s2s, inv, cnt4 = ops.moe_init_routing(idx4_d, E4)
             ts = hip_time(lambda: ops.moe_init_routing(idx4_d, E4))
             qa = torch.empty((rows4, K4), dtype=torch.uint8, device=dev)
-            qs = torch.empty((rows4, K4 // 32), dtype=torch.uint8, device=dev)
+            # scale rows at the pitch the FFN chain uses (whole 128-byte lines: 256 bytes for K/32 = 224 scale bytes)
+            sp4 = ops.ffn_workspace_layout(T4, K4, N4, E4, TOP4)["a_scales_pitch"]
+            qs = torch.empty((rows4, sp4), dtype=torch.uint8, device=dev)
             st = torch.cuda.current_stream().cuda_stream
             tqs = hip_time(lambda: lib.cmx_quant_scatter(x4.data_ptr(), K4, inv.data_ptr(), qa.data_ptr(), K4, qs.data_ptr(),
-                                                         K4 // 32, T4, K4, TOP4, st))
+                                                         sp4, T4, K4, TOP4, st))
             b_qs = T4 * K4 * 2 + rows4 * (K4 + K4 // 32)
             y4 = torch.randn((rows4, K4), generator=g, device=dev).to(torch.bfloat16)
             tc4 = hip_time(lambda: ops.moe_token_unpermute(y4, inv, p4_d))

@@ -23,7 +23,7 @@ u32, i32, u64, sz = C.c_uint32, C.c_int, C.c_uint64, C.c_size_t
 class FfnWorkspaceLayout(C.Structure):
     _fields_ = [(n, C.c_size_t) for n in (
         "src2sorted", "sorted2src", "counts", "routing_scratch", "gmm_meta",
-        "a_codes", "a_scales", "act_codes", "act_scales", "y", "total")]
+        "a_codes", "a_scales", "act_codes", "act_scales", "y", "total", "a_scales_pitch")]
 
 
 # name -> (restype, argtypes); every symbol include/catccos_mx.h declares

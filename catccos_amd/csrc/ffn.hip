@@ -38,7 +38,10 @@ void layout(uint32_t m, uint32_t k, uint32_t n, uint32_t experts, uint32_t top_k
     L->routing_scratch = take(cmx_moe_routing_workspace_bytes((uint32_t)rows, experts));
     L->gmm_meta = take(2 * cmx_mx_gmm_workspace_bytes(experts));
     L->a_codes = take(rows * k);
-    L->a_scales = take(rows * scale_cols(k));
+    // scale rows of the dispatched tokens at a pitch of whole 128-byte lines: the scatter then writes every line of
+    // this array whole
+    L->a_scales_pitch = round_up(scale_cols(k), 128);
+    L->a_scales = take(rows * (size_t)L->a_scales_pitch);
     L->act_codes = take(rows * (n / 2));
     L->act_scales = take(rows * scale_cols(n / 2));
     L->y = take(rows * k * 2);
@@ -105,9 +108,10 @@ extern "C" int catccos_ascend950_dispatch_ffn_combine(uint32_t blockDim, cmx_str
     int rc = cmx_moe_init_routing(reinterpret_cast<const int32_t*>(expertIdx), m, topK, localExperts, sorted2src,
                                   src2sorted, counts, workspace + L.routing_scratch, stream);
     if (rc != CMX_OK) return rc;
-    rc = cmx_quant_scatter(x, k, src2sorted, a_codes, k, a_scales, scale_cols(k), m, k, topK, stream);
+    const uint32_t ld_as = (uint32_t)L.a_scales_pitch;
+    rc = cmx_quant_scatter(x, k, src2sorted, a_codes, k, a_scales, ld_as, m, k, topK, stream);
     if (rc != CMX_OK) return rc;
-    rc = cmx_mx_gmm_swiglu_quant(a_codes, k, a_scales, scale_cols(k), w1, w1Scale, act_codes, n / 2, act_scales,
+    rc = cmx_mx_gmm_swiglu_quant(a_codes, k, a_scales, ld_as, w1, w1Scale, act_codes, n / 2, act_scales,
                                  scale_cols(n / 2), nullptr, counts, localExperts, rows, n, k, meta1, stream);
     if (rc != CMX_OK) return rc;
     rc = cmx_mx_gmm(act_codes, n / 2, act_scales, scale_cols(n / 2), w2, w2Scale, y, k, counts, localExperts, rows, k,

@@ -216,7 +216,92 @@ __global__ __launch_bounds__(256) void quant_scatter_kernel(const uint16_t* __re
     }
 }
 
+// One workgroup per token: the same two-lanes-per-block arithmetic in passes of 128 blocks, but the token's scale
+// bytes are collected in LDS and every destination gets them as one run of 16-byte stores covering `scale_run` bytes
+// (the scale row, its padding column and zeros up to a multiple of 16, or up to the whole pitch): with a pitch of a
+// whole number of 128-byte lines no line of the scale array is ever written in part.  k <= 32768.
+__global__ __launch_bounds__(256) void quant_scatter_row_kernel(const uint16_t* __restrict__ x, uint32_t ld_x,
+                                                                 const int32_t* __restrict__ src2sorted,
+                                                                 uint8_t* __restrict__ out_codes, uint32_t ld_out,
+                                                                 uint8_t* __restrict__ out_scales, uint32_t ld_outs, uint32_t top_k,
+                                                                 uint32_t nb, uint32_t scale_run) {
+    __shared__ __attribute__((aligned(16))) uint8_t s_scale[1024 + 16];
+    const uint32_t row = blockIdx.x, h = threadIdx.x & 1u;
+    const uint16_t* xrow = x + (size_t)row * ld_x;
+    // zeros behind the scale bytes, 127 in the padding column of an odd count
+    for (uint32_t i = nb + threadIdx.x; i < scale_run; i += 256) s_scale[i] = (i == nb && (nb & 1u)) ? 127 : 0;
+    for (uint32_t r0 = 0; r0 < top_k; r0 += 8) {
+        int32_t dst[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) dst[j] = r0 + j < top_k ? src2sorted[(size_t)row * top_k + r0 + j] : -1;
+        for (uint32_t kb0 = 0; kb0 < nb; kb0 += 256) {                 // two passes of 128 blocks in flight together
+            uint4 raw[2][2];
+#pragma unroll
+            for (int it = 0; it < 2; ++it) {
+                const uint32_t kb = kb0 + it * 128 + (threadIdx.x >> 1);
+                raw[it][0] = raw[it][1] = make_uint4(0, 0, 0, 0);
+                if (kb < nb) {
+                    raw[it][0] = *reinterpret_cast<const uint4*>(xrow + kb * 32 + h * 16);
+                    raw[it][1] = *reinterpret_cast<const uint4*>(xrow + kb * 32 + h * 16 + 8);
+                }
+            }
+#pragma unroll
+            for (int it = 0; it < 2; ++it) {
+                const uint32_t kb = kb0 + it * 128 + (threadIdx.x >> 1);
+                const uint32_t d0[4] = {raw[it][0].x, raw[it][0].y, raw[it][0].z, raw[it][0].w};
+                const uint32_t d1[4] = {raw[it][1].x, raw[it][1].y, raw[it][1].z, raw[it][1].w};
+                uint32_t a0[4], a1[4];
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    a0[i] = d0[i] & 0x7FFF7FFFu;
+                    a1[i] = d1[i] & 0x7FFF7FFFu;
+                }
+                uint32_t m = pk_max_u16(pk_max_u16(pk_max_u16(a0[0], a0[1]), pk_max_u16(a0[2], a0[3])),
+                                        pk_max_u16(pk_max_u16(a1[0], a1[1]), pk_max_u16(a1[2], a1[3])));
+                m = pk_max_u16(m, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)m, 0xB1, 0xF, 0xF, true));      // the block's other lane
+                const uint32_t amax = max(m & 0xFFFFu, m >> 16);
+                const int e = block_exp_from_bf16_amax(amax, kEmaxE4M3);
+                const uint32_t lim = (((uint32_t)(e + kEmaxE4M3 + 127) << 7) | 0x60u) * 0x10001u;
+                const float scale = __uint_as_float((uint32_t)(e + 127) << 23);
+                uint32_t c0[4], c1[4];
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    c0[i] = pk_min_u16(a0[i], lim) | (d0[i] & 0x80008000u);
+                    c1[i] = pk_min_u16(a1[i], lim) | (d1[i] & 0x80008000u);
+                }
+                uint32_t w0 = cvt_scaled_pk4<CMX_FMT_E4M3>(c0[0], c0[1], scale), w1 = cvt_scaled_pk4<CMX_FMT_E4M3>(c0[2], c0[3], scale);
+                uint32_t w2 = cvt_scaled_pk4<CMX_FMT_E4M3>(c1[0], c1[1], scale), w3 = cvt_scaled_pk4<CMX_FMT_E4M3>(c1[2], c1[3], scale);
+                if (amax >= 0x7F80u) {                                  // Inf / NaN in the block (rare)
+                    patch_nonfinite_fp8<CMX_FMT_E4M3, false>(d0, w0, w1);
+                    patch_nonfinite_fp8<CMX_FMT_E4M3, false>(d1, w2, w3);
+                }
+                if (kb >= nb) continue;
+                if (r0 == 0 && h == 0) s_scale[kb] = (uint8_t)(e + 127);
+                const uint4 codes = make_uint4(w0, w1, w2, w3);
+#pragma unroll
+                for (int j = 0; j < 8; ++j)
+                    if (dst[j] >= 0) *reinterpret_cast<uint4*>(out_codes + (size_t)dst[j] * ld_out + kb * 32 + h * 16) = codes;
+            }
+        }
+        __syncthreads();                                                // the token's scale bytes are complete
+        for (uint32_t c = threadIdx.x; c < 8 * (scale_run / 16); c += 256) {
+            const uint32_t j = c / (scale_run / 16), q = c - j * (scale_run / 16);
+            const int32_t d = j == 0 ? dst[0] : j == 1 ? dst[1] : j == 2 ? dst[2] : j == 3 ? dst[3] : j == 4 ? dst[4] : j == 5 ? dst[5] : j == 6 ? dst[6] : dst[7];
+            if (d >= 0) *reinterpret_cast<uint4*>(out_scales + (size_t)d * ld_outs + q * 16) = *reinterpret_cast<const uint4*>(s_scale + q * 16);
+        }
+    }
+}
+
 // ---- weighted top-k combine -----------------------------------------------------------------------
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ uint4 load_stream16(const void* p) {
+    const u32x4 v = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p));
+    return make_uint4(v[0], v[1], v[2], v[3]);
+}
+__device__ __forceinline__ void store_stream16(void* p, uint4 v) {
+    __builtin_nontemporal_store((u32x4){v.x, v.y, v.z, v.w}, reinterpret_cast<u32x4*>(p));
+}
+
 // Rows of whole 16-byte vectors: one lane per (token, 8 hidden elements), items numbered token-major, so that
 // every lane has the same amount of work whatever the hidden size.  A lane reads its token's eight row indices
 // and weights (the same addresses across most of a wavefront: one transaction), issues the eight 16-byte gathers
@@ -248,7 +333,9 @@ __global__ __launch_bounds__(256) void unpermute_vec_kernel(const uint16_t* __re
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
             ok[j] = r[j] >= 0 && (uint32_t)r[j] < rows;
-            raw[j] = ok[j] ? *reinterpret_cast<const uint4*>(y + (size_t)r[j] * ld_y + v * 8) : make_uint4(0, 0, 0, 0);
+            // every row is read exactly once: a streaming (non-temporal) load keeps it out of the way of the others
+            // (measured: 183 us instead of 209 us at 8192 tokens x top-8 x 7168)
+            raw[j] = ok[j] ? load_stream16(y + (size_t)r[j] * ld_y + v * 8) : make_uint4(0, 0, 0, 0);
         }
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
@@ -268,7 +355,7 @@ __global__ __launch_bounds__(256) void unpermute_vec_kernel(const uint16_t* __re
     uint32_t o[4];
 #pragma unroll
     for (int i = 0; i < 4; ++i) o[i] = f32_to_bf16(acc[2 * i]) | (f32_to_bf16(acc[2 * i + 1]) << 16);
-    *reinterpret_cast<uint4*>(out + (size_t)t * ld_out + v * 8) = make_uint4(o[0], o[1], o[2], o[3]);
+    store_stream16(out + (size_t)t * ld_out + v * 8, make_uint4(o[0], o[1], o[2], o[3]));
 }
 
 // Any hidden size (the ragged tail element by element): one workgroup per token; a lane owns 8 consecutive hidden
@@ -446,10 +533,22 @@ extern "C" int cmx_quant_scatter(const void* x, uint32_t ld_x, const int32_t* sr
     const uint32_t nb = k / 32;
     CMX_REQUIRE((uint64_t)tokens * nb < (1ull << 32), "too many blocks for one launch");
     const uint32_t total = tokens * nb;
-    const bool vec_scales = nb % 4 == 0 && ld_outs % 4 == 0 && (reinterpret_cast<uintptr_t>(out_scales) & 3u) == 0;
-    const dim3 grid(ceil_div(total, 128));
     const uint16_t* xp = static_cast<const uint16_t*>(x);
     hipStream_t s = static_cast<hipStream_t>(stream);
+    // Scale rows that can be written in 16-byte pieces take the row-wise kernel: the row, its padding column and zeros
+    // up to a multiple of 16 bytes -- or up to the whole pitch when that is the next multiple of 128 (then every
+    // 128-byte line of the scale array is written whole).  Bytes of a row behind its scale_cols(k) columns belong
+    // to the pitch, not to the data, and callers must not keep anything there.
+    const uint32_t run16 = round_up(scale_cols(k), 16);
+    if (ld_outs % 16 == 0 && aligned16(out_scales) && run16 <= ld_outs && nb <= 1024) {
+        const uint32_t run = ld_outs == round_up(scale_cols(k), 128) ? ld_outs : run16;
+        hipLaunchKernelGGL(quant_scatter_row_kernel, dim3(tokens), dim3(256), 0, s, xp, ld_x, src2sorted, out_codes, ld_out,
+                           out_scales, ld_outs, top_k, nb, run);
+        CMX_LAUNCH_CHECK();
+        return CMX_OK;
+    }
+    const bool vec_scales = nb % 4 == 0 && ld_outs % 4 == 0 && (reinterpret_cast<uintptr_t>(out_scales) & 3u) == 0;
+    const dim3 grid(ceil_div(total, 128));
     if (vec_scales)
         hipLaunchKernelGGL((quant_scatter_kernel<true>), grid, dim3(256), 0, s, xp, ld_x, src2sorted, out_codes, ld_out,
                            out_scales, ld_outs, tokens, k, top_k, nb, total);

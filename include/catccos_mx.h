@@ -267,7 +267,9 @@ int cmx_moe_init_routing(const int32_t* expert_idx, uint32_t tokens, uint32_t to
  *
  *   x           bf16 [tokens, k]
  *   src2sorted  int32 [tokens*top_k]; negative destinations are skipped
- *   out_codes   row r at out_codes + r*ld_out (16-byte aligned rows);  out_scales row r at out_scales + r*ld_outs
+ *   out_codes   row r at out_codes + r*ld_out (16-byte aligned rows);  out_scales row r at out_scales + r*ld_outs.
+ *               Bytes of a scale row behind its RoundUp2(k/32) columns, up to the pitch, may be overwritten with zeros
+ *               (scale rows are written in 16-byte pieces, whole 128-byte lines when the pitch is the next multiple of 128).
  * The reference's packed wire row [codes k | scales RoundUp2(k/32) | pad to 32 B] is the case
  * out_scales = out_codes + k, ld_out = ld_outs = cmx_packed_row_bytes(k).
  * ---------------------------------------------------------------------------------------- */
@@ -315,6 +317,7 @@ typedef struct cmx_ffn_workspace_layout {
     size_t src2sorted, sorted2src, counts, routing_scratch, gmm_meta;
     size_t a_codes, a_scales, act_codes, act_scales, y;
     size_t total;
+    size_t a_scales_pitch; /* bytes between the scale rows at a_scales (a multiple of 128, >= RoundUp2(k/32)) */
 } cmx_ffn_workspace_layout;
 int cmx_ffn_workspace_layout_get(uint32_t m, uint32_t k, uint32_t n, uint32_t localExperts, uint32_t topK,
                                  cmx_ffn_workspace_layout* layout);

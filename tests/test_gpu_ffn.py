@@ -48,7 +48,8 @@ def test_ffn_vs_oracle(tokens, k, n, experts, top_k):
     assert np.array_equal(w[lay["sorted2src"]:lay["sorted2src"] + rows * 4].view(np.int32), st["sorted2src"])
     assert np.array_equal(w[lay["counts"]:lay["counts"] + experts * 4].view(np.int32), st["counts"])
     assert np.array_equal(w[lay["a_codes"]:lay["a_codes"] + rows * k].reshape(rows, k), st["aq"])
-    assert np.array_equal(w[lay["a_scales"]:lay["a_scales"] + rows * (k // 32)].reshape(rows, k // 32), st["asc"])
+    pitch = lay["a_scales_pitch"]                     # scale rows sit at a pitch of whole 128-byte lines
+    assert np.array_equal(w[lay["a_scales"]:lay["a_scales"] + rows * pitch].reshape(rows, pitch)[:, :k // 32], st["asc"])
     # stage by stage on the kernel's own intermediates
     half = n // 2
     qa = w[lay["act_codes"]:lay["act_codes"] + rows * half].reshape(rows, half)

@@ -167,7 +167,7 @@ def test_config4_ffn_full_size():
     cnts = _np(view("counts", E * 4).view(torch.int32))
     assert np.array_equal(cnts, np.bincount(idx_h.reshape(-1), minlength=E))
     a_codes = view("a_codes", rows * K).view(rows, K)
-    a_scales = view("a_scales", rows * (K // 32)).view(rows, K // 32)
+    a_scales = view("a_scales", rows * lay["a_scales_pitch"]).view(rows, lay["a_scales_pitch"])[:, :K // 32]
     act_codes = view("act_codes", rows * half).view(rows, half)
     act_scales = view("act_scales", rows * (half // 32)).view(rows, half // 32)
     y = view("y", rows * K * 2).view(torch.int16).view(rows, K)
