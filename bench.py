@@ -43,7 +43,7 @@ def main() -> int:
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=30,
                     help="untimed launches first; the launch time keeps falling for about 25 launches after an idle GPU")
-    ap.add_argument("--only", type=str, default="", help="comma list of extras: quant,gemm,ffn,fp4,int8,routing,copycal (default: all but copycal)")
+    ap.add_argument("--only", type=str, default="", help="comma list of extras: quant,gemm,ffn,fp4,int8,routing,idle,copycal (default: all but copycal)")
     ap.add_argument("--no-extras", action="store_true")
     ap.add_argument("--no-cpu", action="store_true")
     args = ap.parse_args()
@@ -63,8 +63,9 @@ def main() -> int:
     torch.cuda.set_device(dev)
     K_STEPS, WARM = args.steps, args.warmup
 
-    def hip_time(fn, steps=K_STEPS, warm=WARM):
-        """Average duration (s) of fn() over `steps` launches, HIP events on the launch stream."""
+    def hip_time(fn, steps=K_STEPS, warm=max(WARM, 25)):
+        """Average duration (s) of fn() over `steps` launches, HIP events on the launch stream (the extras: at least 25
+        untimed launches first, past the power-management ramp that follows a change of load)."""
         for _ in range(warm):
             fn()
         torch.cuda.synchronize()
@@ -108,70 +109,61 @@ def main() -> int:
     def step():
         ops.mx_gmm_swiglu_quant(a_codes, a_scales, w1, w1s, counts, H, workspace=gws, outs=(act_codes, act_scales))
 
-    # one timed region, measured twice: host clock bracketed by synchronize (-> value) and HIP events recorded on
-    # the launch stream around the same K launches (-> roofline.achieved)
-    for _ in range(WARM):
-        step()
-    torch.cuda.synchronize()
-    ev0 = torch.cuda.Event(enable_timing=True)
-    ev1 = torch.cuda.Event(enable_timing=True)
-    t0 = time.perf_counter()
-    ev0.record()
-    for _ in range(K_STEPS):
-        step()
-    ev1.record()
-    torch.cuda.synchronize()
-    wall = (time.perf_counter() - t0) / K_STEPS
-    kern = ev0.elapsed_time(ev1) * 1e-3 / K_STEPS
-    flop = 2.0 * rows * H * N
-    value = flop / wall / 1e12
-    log(f"[gmm1+swiglu+requant cfg3] wall {wall*1e6:.1f} us/step, events {kern*1e6:.1f} us -> {flop/kern/1e12:.0f} TFLOP/s")
-    roofline = {"kernel": "mx_gemm_pipe_kernel<E4M3, swiglu+requant epilogue, 256x256 tile, 2x2 wavefronts, persistent> (grouped, config 3; one launch also runs the 1-workgroup gmm_prepare_kernel)", "bound": "mfma",
-                "achieved": flop / kern / 1e12, "peak": MXFP8_PEAK_TFLOPS, "unit": "TFLOP/s",
-                "frac": flop / kern / 1e12 / MXFP8_PEAK_TFLOPS,
-                # HBM-side bytes per launch from the rocprofv3 --pmc runs summarised under profiles/
-                # (FETCH_SIZE 1 151 590 KiB x 2.0 + WRITE_SIZE 118 695 KiB x 1.0, factors from a 1 GiB copy)
-                "traffic": 1151590 * 1024 * 2.0 + 118695 * 1024 * 1.0,
-                "flop_per_launch": flop, "avg_launch_us": kern * 1e6}
+    def time_headline():
+        """One timed region, measured twice: host clock bracketed by synchronize (-> value) and HIP events recorded
+        on the launch stream around the same K launches (-> roofline.achieved)."""
+        for _ in range(WARM):
+            step()
+        torch.cuda.synchronize()
+        ev0 = torch.cuda.Event(enable_timing=True)
+        ev1 = torch.cuda.Event(enable_timing=True)
+        t0 = time.perf_counter()
+        ev0.record()
+        for _ in range(K_STEPS):
+            step()
+        ev1.record()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) / K_STEPS, ev0.elapsed_time(ev1) * 1e-3 / K_STEPS
 
-    # ------------------------------------------------------------------ CPU baseline -----------
-    cpu = None
+    flop = 2.0 * rows * H * N
+
+    # ------------------------------------------------------------------ in-run correctness check ----
+    # Before anything is timed: the benchmarked instantiation (no bf16 output) must give the same codes and scales as
+    # the one that also writes the bf16 SwiGLU values, on every row; those must be what the stand-alone quantizer
+    # makes of that bf16 output; and on sampled rows of the largest expert the bf16 values must agree with the CPU
+    # oracle's golden chain (rtol 2e-2) and the codes with the oracle quantizer, bit for bit.
+    step()
+    chk_codes, chk_scales, chk_act = ops.mx_gmm_swiglu_quant(a_codes, a_scales, w1, w1s, counts, H, want_bf16=True)
+    if not (torch.equal(chk_codes, act_codes) and torch.equal(chk_scales, act_scales)):
+        log("bench.py: the benchmarked kernel disagrees with its bf16-output variant")
+        return 4
+    hq, hs = ops.mx_quant(chk_act, "E4M3", "rne")
+    if not (torch.equal(hq, act_codes) and torch.equal(hs, act_scales)):
+        log("bench.py: requantised codes are not what the quantizer makes of the kernel's bf16 output")
+        return 4
     if not args.no_cpu:
         from oracle import mx_oracle as O
-        sample_groups = [int(i) for i in np.argsort(-counts_h)[:8]]     # the 8 largest experts, up to 2048 rows each
-        cap = 2048
-        off = np.concatenate([[0], np.cumsum(counts_h)])
-        a_h, as_h = [], []
-        cnt = []
-        for gi in sample_groups:
-            r = min(cap, int(counts_h[gi]))
-            a_h.append(a_codes[off[gi]:off[gi] + r].cpu().numpy())
-            as_h.append(a_scales[off[gi]:off[gi] + r].cpu().numpy())
-            cnt.append(r)
-        a_h, as_h = np.concatenate(a_h), np.concatenate(as_h)
-        w_h = w1[sample_groups].cpu().numpy()
-        ws_h = w1s[sample_groups].cpu().numpy()
-        O.gmm1_swiglu_quant(a_h[:64], as_h[:64], w_h[:2], ws_h[:2], [32, 32])        # warm-up
-        reps = []
-        for _ in range(3):
-            t0 = time.perf_counter()
-            O.gmm1_swiglu_quant(a_h, as_h, w_h, ws_h, cnt)
-            reps.append(time.perf_counter() - t0)
-        tc = float(np.median(reps))
-        cflop = 2.0 * sum(cnt) * H * N
-        cores = len(os.sched_getaffinity(0))
-        omp = os.environ.get("OMP_NUM_THREADS")
-        if omp and omp.isdigit():
-            cores = min(cores, int(omp))
-        cpu = {"value": cflop / tc / 1e12, "unit": "TFLOP/s", "cores": cores, "kind": "port",
-               "sample": f"numpy oracle gmm1_swiglu_quant on {len(cnt)} experts x {cnt} rows (K={H}, N={N}), "
-                         f"median of 3 = {tc:.2f} s; includes dequantising operands to fp32"}
-        log(f"[cpu baseline] {cpu['value']*1e3:.1f} GFLOP/s on {cores} threads ({tc:.2f} s)")
-        del a_h, as_h, w_h, ws_h
+        e_big = int(np.argmax(counts_h))
+        off_h = np.concatenate([[0], np.cumsum(counts_h)])
+        pick = off_h[e_big] + np.array([0, 1, counts_h[e_big] // 2, counts_h[e_big] - 1])
+        pk = torch.from_numpy(pick).to(dev)
+        _, act_g, _, _ = O.gmm1_swiglu_quant(a_codes[pk].cpu().numpy(), a_scales[pk].cpu().numpy(), w1[e_big:e_big + 1].cpu().numpy(),
+                                             w1s[e_big:e_big + 1].cpu().numpy(), [len(pick)])
+        got_act = chk_act[pk].view(torch.int16).cpu().numpy().view(np.uint16)
+        gold_act = O.bf16_bits_to_f32(act_g)
+        err = np.abs(O.bf16_bits_to_f32(got_act) - gold_act)
+        oq, osc = O.mx_quant_bf16(got_act, "E4M3", "rne")
+        if (err > 1e-3 + 2e-2 * np.abs(gold_act)).any() or not np.array_equal(oq, act_codes[pk].cpu().numpy()) \
+                or not np.array_equal(osc, act_scales[pk].cpu().numpy()):
+            log(f"bench.py: sampled rows disagree with the CPU oracle (max abs err {err.max():.4g})")
+            return 4
+        log(f"[check] codes/scales identical across instantiations and to the quantizer on all {rows} rows; "
+            f"4 sampled rows vs CPU oracle: max abs err {err.max():.3g}")
+    del chk_codes, chk_scales, chk_act, hq, hs
 
     # ------------------------------------------------------------------ extras -----------------
     extra = {}
-    want = set(x for x in args.only.split(",") if x) or {"quant", "gemm", "ffn", "fp4", "int8", "routing"}
+    want = set(x for x in args.only.split(",") if x) or {"quant", "gemm", "ffn", "fp4", "int8", "routing", "idle"}
     if args.no_extras:
         want = set()
 
@@ -313,10 +305,110 @@ def main() -> int:
             fl4 = 2.0 * rows4 * K4 * (N4 + N4 // 2)
             by4 = float(w14.numel() + w14s.numel() + w24.numel() + w24s.numel()) + T4 * K4 * 2 \
                 + 2 * rows4 * (K4 + K4 // 32) + 2 * rows4 * (N4 // 2 + N4 // 64) + 2 * rows4 * K4 * 2 + T4 * K4 * 2
-            extra["moe_ffn_cfg4"] = {"ms": tf * 1e3, "tflops": fl4 / tf / 1e12, "mfma_frac": fl4 / tf / 1e12 / MXFP8_PEAK_TFLOPS,
+            # the same chain stage by stage (the C entry points the FFN calls, in its order, on its kind of buffers),
+            # HIP events between the stages: what each kernel takes inside the chain, where it follows other work
+            # instead of a copy of itself
+            lay4 = ops.ffn_workspace_layout(T4, K4, N4, E4, TOP4)
+            sp = lay4["a_scales_pitch"]
+            ac = torch.empty((rows4, K4), dtype=torch.uint8, device=dev)
+            asc = torch.empty((rows4, sp), dtype=torch.uint8, device=dev)
+            hc = torch.empty((rows4, N4 // 2), dtype=torch.uint8, device=dev)
+            hs = torch.empty((rows4, ops.scale_cols(N4 // 2)), dtype=torch.uint8, device=dev)
+            yy = torch.empty((rows4, K4), dtype=torch.bfloat16, device=dev)
+            gw1, gw2 = ops.gmm_workspace(E4, dev), ops.gmm_workspace(E4, dev)
+            st4 = torch.cuda.current_stream().cuda_stream
+            names = ["expert_sort", "quant_scatter", "gmm1_swiglu_requant", "gmm2", "unpermute_combine"]
+            acc_ms = [0.0] * 5
+            reps = max(3, K_STEPS // 4)
+            for rep in range(reps + 2):
+                evs = [torch.cuda.Event(enable_timing=True) for _ in range(6)]
+                evs[0].record()
+                s2s4, inv4, cnt4b = ops.moe_init_routing(idx4_d, E4)
+                evs[1].record()
+                lib.cmx_quant_scatter(x4.data_ptr(), K4, inv4.data_ptr(), ac.data_ptr(), K4, asc.data_ptr(), sp, T4, K4, TOP4, st4)
+                evs[2].record()
+                ops.mx_gmm_swiglu_quant(ac, asc, w14, w14s, cnt4b, K4, workspace=gw1, outs=(hc, hs))
+                evs[3].record()
+                ops.mx_gmm(hc, hs, w24, w24s, cnt4b, N4 // 2, "E4M3", "bf16", c=yy, workspace=gw2)
+                evs[4].record()
+                ops.moe_token_unpermute(yy, inv4, p4_d)
+                evs[5].record()
+                torch.cuda.synchronize()
+                if rep >= 2:
+                    for i in range(5):
+                        acc_ms[i] += evs[i].elapsed_time(evs[i + 1]) / reps
+            b_qs4 = T4 * K4 * 2 + rows4 * (K4 + K4 // 32)
+            b_c4 = rows4 * K4 * 2 + T4 * K4 * 2
+            stages = {n: {"us": acc_ms[i] * 1e3} for i, n in enumerate(names)}
+            stages["quant_scatter"].update({"hbm_frac": b_qs4 / (acc_ms[1] * 1e-3) / 1e9 / HBM_PEAK_GBS})
+            stages["unpermute_combine"].update({"hbm_frac": b_c4 / (acc_ms[4] * 1e-3) / 1e9 / HBM_PEAK_GBS})
+            log("[moe ffn cfg4 stages] " + ", ".join(f"{n} {v['us']:.0f} us" for n, v in stages.items()))
+            del ac, asc, hc, hs, yy
+            extra["moe_ffn_cfg4"] = {"ms": tf * 1e3, "stages_in_chain": stages, "tflops": fl4 / tf / 1e12, "mfma_frac": fl4 / tf / 1e12 / MXFP8_PEAK_TFLOPS,
                                      "algorithmic_GB": by4 / 1e9, "hbm_GBs": by4 / tf / 1e9, "hbm_frac": by4 / tf / 1e9 / HBM_PEAK_GBS,
                                      "tokens_per_s": T4 / tf}
             log(f"[moe ffn cfg4] {tf*1e3:.3f} ms -> {fl4/tf/1e12:.0f} TFLOP/s, {by4/tf/1e9:.0f} GB/s algorithmic")
+
+    # ------------------------------------------------------------------ headline timing ---------
+    # The extras above ran first, so this is a GPU that has been busy, as it is in a training or serving job.  (After
+    # an idle period the first ~25 launches of an MFMA-bound kernel run up to 30 % slower while the power management
+    # settles: extra.after_idle records that case.)
+    wall, kern = time_headline()
+    value = flop / wall / 1e12
+    log(f"[gmm1+swiglu+requant cfg3] wall {wall*1e6:.1f} us/step, events {kern*1e6:.1f} us -> {flop/kern/1e12:.0f} TFLOP/s")
+    traffic = None
+    tpath = os.path.join(ROOT, "profiles", "traffic_config3.json")
+    if os.path.exists(tpath):
+        # HBM-side bytes per launch from the rocprofv3 --pmc runs summarised next to that file (FETCH_SIZE and
+        # WRITE_SIZE scaled by what the same counters read for a 1 GiB copy); profiled, not measured in this run
+        with open(tpath) as f:
+            traffic = json.load(f).get("traffic_bytes_per_launch")
+    roofline = {"kernel": "mx_gemm_pipe_kernel<E4M3, swiglu+requant epilogue, 256x256 tile, 2x2 wavefronts, persistent> (grouped, config 3; one launch also runs the 1-workgroup gmm_prepare_kernel)", "bound": "mfma",
+                "achieved": flop / kern / 1e12, "peak": MXFP8_PEAK_TFLOPS, "unit": "TFLOP/s",
+                "frac": flop / kern / 1e12 / MXFP8_PEAK_TFLOPS, "traffic": traffic,
+                "flop_per_launch": flop, "avg_launch_us": kern * 1e6}
+    if "idle" in want:
+        time.sleep(3.0)
+        saved = (WARM, K_STEPS)
+        w_idle, k_idle = time_headline()
+        extra["after_idle"] = {"idle_s": 3.0, "warmup": WARM, "steps": K_STEPS, "avg_launch_us": k_idle * 1e6,
+                               "note": "the same timed region started 3 s after the GPU went idle"}
+        log(f"[after 3 s idle] events {k_idle*1e6:.1f} us")
+
+    # ------------------------------------------------------------------ CPU baseline -----------
+    cpu = None
+    if not args.no_cpu:
+        from oracle import mx_oracle as O
+        sample_groups = [int(i) for i in np.argsort(-counts_h)[:8]]     # the 8 largest experts, up to 2048 rows each
+        cap = 2048
+        off = np.concatenate([[0], np.cumsum(counts_h)])
+        a_h, as_h = [], []
+        cnt = []
+        for gi in sample_groups:
+            r = min(cap, int(counts_h[gi]))
+            a_h.append(a_codes[off[gi]:off[gi] + r].cpu().numpy())
+            as_h.append(a_scales[off[gi]:off[gi] + r].cpu().numpy())
+            cnt.append(r)
+        a_h, as_h = np.concatenate(a_h), np.concatenate(as_h)
+        w_h = w1[sample_groups].cpu().numpy()
+        ws_h = w1s[sample_groups].cpu().numpy()
+        O.gmm1_swiglu_quant(a_h[:64], as_h[:64], w_h[:2], ws_h[:2], [32, 32])        # warm-up
+        reps = []
+        for _ in range(3):
+            t0 = time.perf_counter()
+            O.gmm1_swiglu_quant(a_h, as_h, w_h, ws_h, cnt)
+            reps.append(time.perf_counter() - t0)
+        tc = float(np.median(reps))
+        cflop = 2.0 * sum(cnt) * H * N
+        cores = len(os.sched_getaffinity(0))
+        omp = os.environ.get("OMP_NUM_THREADS")
+        if omp and omp.isdigit():
+            cores = min(cores, int(omp))
+        cpu = {"value": cflop / tc / 1e12, "unit": "TFLOP/s", "cores": cores, "kind": "port",
+               "sample": f"numpy oracle gmm1_swiglu_quant on {len(cnt)} experts x {cnt} rows (K={H}, N={N}), "
+                         f"median of 3 = {tc:.2f} s; includes dequantising operands to fp32"}
+        log(f"[cpu baseline] {cpu['value']*1e3:.1f} GFLOP/s on {cores} threads ({tc:.2f} s)")
+        del a_h, as_h, w_h, ws_h
 
     line = {
         "metric": "MXFP8 GMM TFLOP/s (% MFMA peak); MX-quant GB/s (% HBM peak), 1 GPU",
