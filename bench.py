@@ -215,12 +215,34 @@ def main() -> int:
         # the same B stored [K, N] with scales [K/64, N, 2]: the layout pass alone (one read + one write of B)
         bt = b2.t().contiguous()
         bts = b2s.reshape(N2, K2 // 64, 2).permute(1, 0, 2).contiguous()
-        tl = hip_time(lambda: ops.mx_to_k_major(bt, bts, K2, N2))
+        bk = torch.empty((N2, K2), dtype=torch.uint8, device=dev)
+        bks = torch.empty((N2, K2 // 32), dtype=torch.uint8, device=dev)
+        st2 = torch.cuda.current_stream().cuda_stream
+        tl = hip_time(lambda: lib.cmx_mx_to_k_major(bt.data_ptr(), N2, bts.data_ptr(), bk.data_ptr(), K2, bks.data_ptr(), K2 // 32,
+                                                    K2, N2, 1, st2))
         bytes_l = 2 * (N2 * K2 + N2 * K2 // 32)
-        extra["mx_to_k_major_cfg2_B"] = {"kernel": "mx_to_k_major_kernel", "bound": "hbm", "achieved": bytes_l / tl / 1e9,
+        # a 30 MB operand is gone in a dozen microseconds: a plain device copy of the same bytes is the yardstick there;
+        # the sixteen experts of config 3's W1 (485 MB) show the rate of the kernel itself
+        flat = torch.empty(bytes_l // 2, dtype=torch.uint8, device=dev)
+        flat2 = torch.empty_like(flat)
+        tcp = hip_time(lambda: flat2.copy_(flat))
+        wt = torch.empty((E, H, N), dtype=torch.uint8, device=dev)
+        wts = torch.empty((E, H // 64, N, 2), dtype=torch.uint8, device=dev)
+        wk = torch.empty((E, N, H), dtype=torch.uint8, device=dev)
+        wks = torch.empty((E, N, H // 32), dtype=torch.uint8, device=dev)
+        tlw = hip_time(lambda: lib.cmx_mx_to_k_major(wt.data_ptr(), N, wts.data_ptr(), wk.data_ptr(), H, wks.data_ptr(), H // 32,
+                                                     H, N, E, st2), steps=max(5, K_STEPS // 2))
+        bytes_w = 2 * E * (N * H + N * H // 32)
+        extra["mx_to_k_major_cfg2_B"] = {"kernel": "mx_to_k_major16_kernel", "bound": "hbm", "achieved": bytes_l / tl / 1e9,
                                          "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": bytes_l / tl / 1e9 / HBM_PEAK_GBS,
-                                         "bytes_per_launch": bytes_l, "avg_launch_us": tl * 1e6}
-        log(f"[mx_to_k_major cfg2 B] {tl*1e6:.1f} us -> {bytes_l/tl/1e9:.0f} GB/s")
+                                         "bytes_per_launch": bytes_l, "avg_launch_us": tl * 1e6,
+                                         "device_copy_of_the_same_bytes_us": tcp * 1e6}
+        extra["mx_to_k_major_cfg3_W1"] = {"kernel": "mx_to_k_major16_kernel", "bound": "hbm", "achieved": bytes_w / tlw / 1e9,
+                                          "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": bytes_w / tlw / 1e9 / HBM_PEAK_GBS,
+                                          "bytes_per_launch": bytes_w, "avg_launch_us": tlw * 1e6}
+        log(f"[mx_to_k_major cfg2 B] {tl*1e6:.1f} us -> {bytes_l/tl/1e9:.0f} GB/s (copy of the same bytes {tcp*1e6:.1f} us); "
+            f"cfg3 W1 {tlw*1e6:.1f} us -> {bytes_w/tlw/1e9:.0f} GB/s")
+        del bk, bks, flat, flat2, wt, wts, wk, wks
         del a2, a2s, b2, b2s, bt, bts
 
     if "int8" in want:
@@ -287,12 +309,37 @@ def main() -> int:
             y4 = torch.randn((rows4, K4), generator=g, device=dev).to(torch.bfloat16)
             tc4 = hip_time(lambda: ops.moe_token_unpermute(y4, inv, p4_d))
             b_c = rows4 * K4 * 2 + T4 * K4 * 2
+
+            def spaced(fn, reps=8):
+                """Average duration (s) of single launches of fn() that each follow a launch of the headline matmul
+                instead of a copy of themselves (HIP events around every launch)."""
+                tot = 0.0
+                for r in range(reps + 2):
+                    step()
+                    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                    e0.record()
+                    fn()
+                    e1.record()
+                    torch.cuda.synchronize()
+                    if r >= 2:
+                        tot += e0.elapsed_time(e1) * 1e-3 / reps
+                return tot
+
+            # back to back, a kernel that writes 486 MB competes with the write-back of its predecessor's lines (the
+            # memory-side cache still holds them); inside the FFN chain it follows a matmul that leaves HBM bandwidth
+            # free.  "frac" is the sustained back-to-back rate, "frac_after_matmul" the rate of a launch placed as in
+            # the chain.
+            tqs_sp = spaced(lambda: lib.cmx_quant_scatter(x4.data_ptr(), K4, inv.data_ptr(), qa.data_ptr(), K4, qs.data_ptr(),
+                                                          sp4, T4, K4, TOP4, st))
+            tc4_sp = spaced(lambda: ops.moe_token_unpermute(y4, inv, p4_d))
             extra["routing_cfg4"] = {
                 "expert_sort_us": ts * 1e6,
                 "quant_scatter": {"bound": "hbm", "achieved": b_qs / tqs / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                                  "frac": b_qs / tqs / 1e9 / HBM_PEAK_GBS, "avg_launch_us": tqs * 1e6},
+                                  "frac": b_qs / tqs / 1e9 / HBM_PEAK_GBS, "avg_launch_us": tqs * 1e6,
+                                  "after_matmul_us": tqs_sp * 1e6, "frac_after_matmul": b_qs / tqs_sp / 1e9 / HBM_PEAK_GBS},
                 "unpermute_combine": {"bound": "hbm", "achieved": b_c / tc4 / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                                      "frac": b_c / tc4 / 1e9 / HBM_PEAK_GBS, "avg_launch_us": tc4 * 1e6}}
+                                      "frac": b_c / tc4 / 1e9 / HBM_PEAK_GBS, "avg_launch_us": tc4 * 1e6,
+                                      "after_matmul_us": tc4_sp * 1e6, "frac_after_matmul": b_c / tc4_sp / 1e9 / HBM_PEAK_GBS}}
             log(f"[routing cfg4] sort {ts*1e6:.1f} us, quant_scatter {b_qs/tqs/1e9:.0f} GB/s, combine {b_c/tc4/1e9:.0f} GB/s")
             del qa, qs, y4
         if "ffn" in want:

@@ -22,6 +22,7 @@ namespace {
 
 constexpr int kLt = 128;                 // tile edge in bytes, both ways
 constexpr int kLtPitch = kLt / 4 + 1;    // LDS row pitch in dwords
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 
 // bytes (i, j) -> (j, i) of the 4 x 4 byte matrix whose rows are r0..r3; c[j] = {r0.j, r1.j, r2.j, r3.j}
 __device__ __forceinline__ void transpose4x4(uint32_t r0, uint32_t r1, uint32_t r2, uint32_t r3, uint32_t (&c)[4]) {
@@ -107,6 +108,65 @@ __global__ __launch_bounds__(256) void mx_to_k_major_kernel(const uint8_t* __res
             }
         }
     }
+}
+
+// The same tile with 16-byte loads, for sources whose rows are 16-byte aligned and whose n is a multiple of 16 (a
+// 16-byte piece is then whole or absent): a thread loads 16 bytes of four consecutive K rows (all four loads in flight
+// before the first use), transposes its four 4 x 4 byte blocks and stages sixteen dwords.  The LDS tile is
+// [n][32 dwords of K] with the dword index XORed by 4 (n / 16): the sixteen lanes-times-rows that write at once differ
+// in n / 16 and in the low K bits and so hit 32 different banks, and the 16-byte runs the store phase reads stay whole.
+// Every byte is touched once, so loads and stores are non-temporal (3 % on 485 MB of weights).
+__global__ __launch_bounds__(256) void mx_to_k_major16_kernel(const uint8_t* __restrict__ src, uint32_t ld_src,
+                                                              const uint8_t* __restrict__ src_scale,
+                                                              uint8_t* __restrict__ dst, uint32_t ld_dst,
+                                                              uint8_t* __restrict__ dst_scale, uint32_t ld_dst_scale,
+                                                              uint32_t k, uint32_t n, uint64_t src_batch,
+                                                              uint64_t dst_batch, uint64_t src_scale_batch,
+                                                              uint64_t dst_scale_batch) {
+    __shared__ __attribute__((aligned(16))) uint32_t tile[kLt * 32];   // [n][(k / 4) ^ swizzle(n)]
+    const uint32_t t = threadIdx.x;
+    const uint32_t n0 = blockIdx.x * kLt, k0 = blockIdx.y * kLt;
+    src += blockIdx.z * src_batch;
+    dst += blockIdx.z * dst_batch;
+
+    // scales first (their loads overlap the tile's): [pair][n][2] -> [n][2 pair + {0, 1}], one 16-bit unit per thread
+    uint32_t sval = 0;
+    const uint32_t s_n = n0 + (t & 127u), s_pair = k0 / 64 + (t >> 7);
+    const bool s_on = src_scale != nullptr && s_n < n && s_pair * 64 < k;
+    if (s_on)
+        sval = *reinterpret_cast<const uint16_t*>(src_scale + blockIdx.z * src_scale_batch + ((size_t)s_pair * n + s_n) * 2);
+
+    const uint32_t nq = t & 7u, kq = t >> 3;          // 16 bytes along N, rows 4 kq .. 4 kq + 3
+    const uint32_t ncol = n0 + 16 * nq;
+    u32x4 r[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const uint32_t kr = k0 + 4 * kq + j;
+        r[j] = u32x4{0, 0, 0, 0};
+        if (kr < k && ncol < n) r[j] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(src + (size_t)kr * ld_src + ncol));
+    }
+#pragma unroll
+    for (int d = 0; d < 4; ++d) {
+        uint32_t c[4];
+        transpose4x4(r[0][d], r[1][d], r[2][d], r[3][d], c);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) tile[(16 * nq + 4 * d + j) * 32 + (kq ^ (4 * nq))] = c[j];
+    }
+    __syncthreads();
+
+    const uint32_t part = t & 7u;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const uint32_t nr = (t >> 3) + 32 * i;
+        const uint32_t kc = k0 + 16 * part;
+        if (n0 + nr < n && kc < k) {
+            const u32x4 q = *reinterpret_cast<const u32x4*>(tile + nr * 32 + ((4 * part) ^ (4 * (nr >> 4))));
+            __builtin_nontemporal_store(q, reinterpret_cast<u32x4*>(dst + (size_t)(n0 + nr) * ld_dst + kc));
+        }
+    }
+    if (s_on)
+        *reinterpret_cast<uint16_t*>(dst_scale + blockIdx.z * dst_scale_batch + (size_t)s_n * ld_dst_scale + 2 * s_pair) =
+            (uint16_t)sval;
 }
 
 // FP4: two codes share a byte along the contiguous axis, so the same change of orientation is a transpose of 4-bit
@@ -231,6 +291,15 @@ int to_k_major(const uint8_t* src, uint32_t ld_src, const uint8_t* src_scale, ui
     CMX_REQUIRE(batch <= 65535u && ceil_div(k, kLt) <= 65535u, "too many tiles for one launch");
     const int vec_in = ld_src % 4 == 0 && (reinterpret_cast<uintptr_t>(src) & 3u) == 0;
     dim3 grid(ceil_div(n, kLt), ceil_div(k, kLt), batch);
+    const bool scales16 = src_scale == nullptr || (((reinterpret_cast<uintptr_t>(src_scale) | reinterpret_cast<uintptr_t>(dst_scale)) & 1u) == 0 &&
+                                                   ld_dst_scale % 2 == 0);
+    if (ld_src % 16 == 0 && aligned16(src) && n % 16 == 0 && scales16) {
+        hipLaunchKernelGGL(mx_to_k_major16_kernel, grid, dim3(256), 0, s, src, ld_src, src_scale, dst, ld_dst, dst_scale,
+                           ld_dst_scale, k, n, (uint64_t)k * ld_src, (uint64_t)n * ld_dst, (uint64_t)(k / 32) * n,
+                           (uint64_t)n * ld_dst_scale);
+        CMX_LAUNCH_CHECK();
+        return CMX_OK;
+    }
     hipLaunchKernelGGL(mx_to_k_major_kernel, grid, dim3(256), 0, s, src, ld_src, src_scale, dst, ld_dst, dst_scale,
                        ld_dst_scale, k, n, (uint64_t)k * ld_src, (uint64_t)n * ld_dst, (uint64_t)(k / 32) * n,
                        (uint64_t)n * ld_dst_scale, vec_in);

@@ -33,7 +33,7 @@ public:
         l.counts = take(experts * sizeof(int32_t));
         l.aCodes = take(rows * t.k);
         l.tokScale = take(rows * sizeof(float));
-        l.gmm = take(cmx_int8_gmm_workspace_bytes(experts, t.n, t.k, 0));
+        l.gmm = take(cmx_int8_gmm_workspace_bytes(experts, t.n, t.k, 1));
         l.total = off;
         return l;
     }
@@ -51,7 +51,13 @@ public:
             std::vector<uint16_t> ones(static_cast<size_t>(t.m) * t.k, 0x3F80);
             a = mxops::DeviceBufferFromValues(ones.data(), aBytes);
         }
-        uint8_t* b = mxops::DeviceBufferFromFile(static_cast<size_t>(t.k) * t.n * experts, fromFiles ? file("b_gm") : "", 1);
+        // b_gm is [E, k, n] on disk; the weights do not change between launches, so they are rewritten K-contiguous
+        // ([E, n, k]) once here and every launch runs with trans_b = 1 (otherwise each call would move them again)
+        uint8_t* bFile = mxops::DeviceBufferFromFile(static_cast<size_t>(t.k) * t.n * experts, fromFiles ? file("b_gm") : "", 1);
+        uint8_t* b = mxrt::DeviceAlloc(static_cast<size_t>(t.k) * t.n * experts);
+        MX_CHECK(cmx_bytes_to_k_major(bFile, t.n, b, t.k, t.k, t.n, static_cast<uint32_t>(experts), nullptr));
+        MX_CHECK(cmx_rt_stream_sync(nullptr));
+        MX_CHECK(cmx_rt_free(bFile));
         uint8_t* scale = nullptr;
         const size_t scaleBytes = static_cast<size_t>(t.n) * experts * sizeof(uint64_t);
         if (fromFiles) {
@@ -87,7 +93,7 @@ public:
         if (rc != CMX_OK) return rc;
         return cmx_int8_gmm_dequant_swiglu(aCodes, t.k, tokScale, reinterpret_cast<const int8_t*>(p.ptrB),
                                            reinterpret_cast<const float*>(p.customPtrs[0]), 2, p.ptrC, t.n / 2, CMX_OUT_BF16, counts,
-                                           experts, rows, t.n, t.k, 0, ws + l.gmm, stream);
+                                           experts, rows, t.n, t.k, 1, ws + l.gmm, stream);
     }
 
     // ---- MX ---------------------------------------------------------------------------------------------
