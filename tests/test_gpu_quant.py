@@ -85,6 +85,35 @@ def test_zero_and_tiny_blocks():
     _check(O.f32_to_bf16_bits(x), "E2M1", "lut")
 
 
+def _with_non_finite(rows, cols, seed):
+    """Seeded activations with +-Inf and NaN (both signs, several payloads) dropped into a sixth of the blocks: alone, together,
+    as the first and the last element of a block, and one block made of nothing else."""
+    xb = W.activations_with_outliers(rows, cols, seed=seed).copy()
+    rng = np.random.default_rng(seed + 1)
+    specials = np.array([0x7F80, 0xFF80, 0x7FC0, 0xFFC0, 0x7F81, 0xFFFF], dtype=np.uint16)
+    nb = (cols + 31) // 32
+    for r in range(rows):
+        for b in rng.choice(nb, size=max(1, nb // 6), replace=False):
+            lo, hi = b * 32, min(cols, b * 32 + 32)
+            pos = rng.choice(np.arange(lo, hi), size=min(hi - lo, int(rng.integers(1, 4))), replace=False)
+            xb[r, pos] = rng.choice(specials, size=pos.size)
+    xb[0, 0] = 0x7F80                     # first element of a block
+    xb[0, min(cols, 32) - 1] = 0xFFC0     # last element of the same block: Inf and NaN together
+    if cols >= 64:
+        xb[rows - 1, 32:64] = 0x7FC0      # a block of NaNs only
+    return xb
+
+
+@pytest.mark.parametrize("fmt,mode", CASES)
+@pytest.mark.parametrize("rows,cols", [(8, 7168), (5, 1000), (3, 96)])
+def test_non_finite_elements_follow_the_golden_rule(fmt, mode, rows, cols):
+    """Inf / NaN elements and blocks: scale bytes 247 / 240 (8-bit formats), 254 / 255 (4-bit formats), Inf to the largest
+    code, NaN to the NaN code or to 0 -- the rule of the reference's generator (gen_mx_quant_allgather_data.py:181-189, 285-288),
+    which the oracle restates and the fixtures made by that generator pin.  (8, 7168) takes the packed bf16 kernel for
+    E4M3 / E5M2 with RNE, the other shapes the general one."""
+    _check(_with_non_finite(rows, cols, 17 * rows + cols), fmt, mode)
+
+
 def test_row_pitches():
     from catccos_amd import _lib
     xb = W.activations_with_outliers(16, 256, seed=5)

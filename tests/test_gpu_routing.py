@@ -54,6 +54,27 @@ def test_quant_scatter_bit_exact(packed):
         assert np.array_equal(host(codes), want[:, :k]) and np.array_equal(host(scales), want[:, k:k + k // 32])
 
 
+@pytest.mark.parametrize("k", [512, 7168, 96])
+def test_quant_scatter_non_finite_tokens_equal_the_quantizer(k):
+    """Tokens with Inf / NaN elements through both scatter kernels (k = 96: scale rows that are not 16-byte aligned take the
+    general kernel) give the rows the stand-alone quantizer and the oracle give."""
+    from catccos_amd import ops
+    from tests.test_gpu_quant import _with_non_finite
+    tokens, top_k = 24, 3
+    xb = _with_non_finite(tokens, k, seed=k)
+    rng = np.random.default_rng(k)
+    inv = rng.permutation(tokens * top_k).astype(np.int32)
+    codes, scales = ops.quant_scatter(bf16_dev(xb), dev(inv), top_k)
+    q, s = O.mx_quant_bf16(xb)
+    got_c, got_s = host(codes), host(scales)
+    nsc = s.shape[1]
+    for t in range(tokens):
+        for r in range(top_k):
+            d = inv[t * top_k + r]
+            assert np.array_equal(got_c[d], q[t]), (t, r)
+            assert np.array_equal(got_s[d, :nsc], s[t]), (t, r)
+
+
 def test_quant_scatter_skips_negative_destinations():
     from catccos_amd import ops
     xb = W.activations_with_outliers(8, 64, seed=9)
