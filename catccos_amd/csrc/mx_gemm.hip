@@ -1033,8 +1033,8 @@ int launch_gemm_dl(const GemmParams& p, uint32_t max_m_tiles, hipStream_t s) {
 
 template <int FMT, int EPI, int TM, int WW, int WM, int NSLOT>
 int launch_gemm_pipe(const GemmParams& p, uint32_t max_m_tiles, hipStream_t s) {
-    // tile ring, scale ring (two-slot kernels: two blocks of 16 bytes per row), next-tile mailbox
-    constexpr size_t smem = NSLOT * (256 + TM) * kSlabBytes + (NSLOT == 2 ? 2 * (256 + TM) * 16 : NSLOT * (256 + TM) * 4) + 16;
+    // tile ring, scale ring (two-slot kernels: two blocks of 16 bytes per row), next-tile mailbox, 256-byte sink of the L2 prefetch loads
+    constexpr size_t smem = NSLOT * (256 + TM) * kSlabBytes + (NSLOT == 2 ? 2 * (256 + TM) * 16 : NSLOT * (256 + TM) * 4) + 512;
     constexpr auto kfn = mx_gemm_pipe_kernel<FMT, EPI, TM, WW, WM, NSLOT>;
     if (int rc = allow_dynamic_lds<kfn, smem>(); rc != CMX_OK) return rc;
     const uint64_t tiles = (uint64_t)max_m_tiles * p.w_tiles;
@@ -1054,7 +1054,7 @@ int launch_gemm_pipe(const GemmParams& p, uint32_t max_m_tiles, hipStream_t s) {
 
 template <int EPI, int WW, int WM>
 int launch_gemm_pipe_fp4(const GemmParams& p, uint32_t max_m_tiles, hipStream_t s) {
-    constexpr size_t smem = 2 * 512 * kSlabBytes + 2 * 512 * 16 + 16;     // tile ring, ring of two scale blocks, next-tile mailbox
+    constexpr size_t smem = 2 * 512 * kSlabBytes + 2 * 512 * 16 + 512;    // tile ring, ring of two scale blocks, next-tile mailbox, sink of the L2 prefetch loads
     constexpr auto kfn = mx_gemm_pipe_fp4_kernel<EPI, WW, WM>;
     if (int rc = allow_dynamic_lds<kfn, smem>(); rc != CMX_OK) return rc;
     const uint64_t tiles = (uint64_t)max_m_tiles * p.w_tiles;

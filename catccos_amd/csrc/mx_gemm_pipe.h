@@ -117,6 +117,22 @@ __device__ __forceinline__ v8i join8(const v4i& lo, const v4i& hi) {
 //           rate, sets the pace.
 __host__ __device__ constexpr bool pipe_is_persistent(int nslot, int epi) { return nslot == 2 && epi != kEpiStore; }
 
+// L2 prefetch distance in slabs for the persistent 2 x 2 kernels (0: none).  While the load stream requests slab q,
+// the workgroup also touches one dword of every 128-byte line of slab q + distance -- of its share of the rows: the
+// workgroups that run side by side on an XCD share operand panels, and each takes the rows congruent to its position
+// in the sharing set, so every line is asked for once per XCD, one to two slab times before the LDS-DMA loads of
+// all sharers want it.  The loads have no register destination (they land in a 256-byte LDS sink nobody reads), and
+// they are issued behind the tile loads of their slab, so every wait in the schedule simply lets two more loads stay
+// in flight.  Loads return in order, so a prefetch must be back within about one and a half slab times or it holds
+// up the tile loads behind it: distances 1 and 2 gain 4-5 % on the Zipf-routed 16-expert problem, 4 gains 2 %, 10
+// nothing (the further ahead, the more often the line comes all the way from HBM).  Prefetching every line of the
+// tile from every workgroup instead (512 instead of 96 lines per slab) costs 20 %: the price is per distinct line,
+// which is why a panel that fewer than four workgroups share is not prefetched at all.
+#ifndef CMX_PIPE_PREFETCH
+#define CMX_PIPE_PREFETCH 2
+#endif
+
+
 template <int FMT, int EPI, int TM, int WW, int WM, int NSLOT>
 __global__ __launch_bounds__(256) void mx_gemm_pipe_kernel(const GemmParams p) {
     static_assert(FMT == CMX_FMT_E4M3 || FMT == CMX_FMT_E5M2, "8-bit element formats only");
@@ -139,6 +155,8 @@ __global__ __launch_bounds__(256) void mx_gemm_pipe_kernel(const GemmParams p) {
     constexpr int kTileLoads = kRows / (8 * NW);              // LDS-DMA loads per wavefront and slab (16 or 12)
     constexpr int kWTileLoads = TW / (8 * NW);                // the first 8 fetch weight rows
     constexpr int kLoadsPerSlab = kTileLoads + 2;             // three-slot kernel: plus one weight and one activation scale load
+    constexpr int kPfAhead = (pipe_is_persistent(NSLOT, EPI) && WW == 2 && WM == 2) ? CMX_PIPE_PREFETCH : 0;
+    constexpr int kPf = kPfAhead > 0 ? 2 : 0;                  // prefetch loads per wavefront and slab
 
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t*)smem;
@@ -169,6 +187,8 @@ __global__ __launch_bounds__(256) void mx_gemm_pipe_kernel(const GemmParams p) {
     Tile tq;                                    // tile of the load stream
     v4i w_rs, a_rs, ws_rs, as_rs;
     uint32_t goff[kTileLoads], sgoff_w, sgoff_a;
+    uint32_t pfoff[2] = {0, 0};                 // prefetch: wavefronts 0, 1 cover the weight rows, 2, 3 the activation rows
+    v4i pf_rs = {0, 0, 0, 0};
     const uint32_t sa_blk = wave % (TM / 64);
     auto make_rsrc = [](const uint8_t* q) -> v4i {
         const uint64_t v = reinterpret_cast<uint64_t>(q);
@@ -217,6 +237,29 @@ __global__ __launch_bounds__(256) void mx_gemm_pipe_kernel(const GemmParams p) {
         // 64*(wave mod TM/64).. (with TM = 128 two wavefronts fetch the same rows to the same place)
         sgoff_w = wrow_of(64 * wave + lane) * p.ld_ws;
         sgoff_a = arow_of(64 * sa_blk + lane) * p.ld_as;
+        if constexpr (kPf > 0) {
+            static_assert(kPf == 0 || (TW == 256 && TM == 256), "the prefetch split assumes 256 + 256 rows");
+            // The workgroups that run side by side on an XCD share operand panels (tile order: bands of m-tiles, m
+            // fastest, across a run of weight tiles): the weight panel with the other m-tiles of the band, the
+            // activation panel with the neighbouring weight tiles.  Each prefetches only its share of a panel's rows
+            // (row = position in the sharing set, modulo its size); the lanes left over repeat the last such row.
+            const uint32_t band = p.row_off != nullptr ? 8u : 4u;
+            const uint32_t mtg = p.row_off != nullptr ? (uint32_t)p.tile_pref[g + 1] - (uint32_t)p.tile_pref[g] : m_tiles_all;
+            const uint32_t mt = tq.mt, b0 = mt / band * band;
+            const uint32_t band_rows = __builtin_amdgcn_readfirstlane(mtg - b0 < band ? mtg - b0 : band);
+            uint32_t nsh_a = 32u / band_rows;
+            nsh_a = __builtin_amdgcn_readfirstlane(nsh_a < p.w_tiles ? nsh_a : p.w_tiles);
+            const uint32_t mod = wave < 2 ? band_rows : nsh_a;
+            const uint32_t sel = __builtin_amdgcn_readfirstlane(wave < 2 ? mt - b0 : wt % nsh_a);
+            const uint32_t last = __builtin_amdgcn_readfirstlane(sel + mod * ((255u - sel) / mod));
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+                uint32_t r = sel + mod * ((2 * (wave & 1u) + j) * 64 + lane);
+                r = (r < 256u && mod >= 4u) ? r : last;      // a panel with fewer than four sharers is left to its own tile loads
+                pfoff[j] = wave < 2 ? mul_lo_u32(wrow_of(r), p.ldw) : mul_lo_u32(arow_of(r), p.lda);
+            }
+            pf_rs = wave < 2 ? w_rs : a_rs;
+        }
     };
     aim_loads_at(tile_id, 0);
     Tile tc = tq;                               // tile of the MFMA stream / epilogue
@@ -231,6 +274,8 @@ __global__ __launch_bounds__(256) void mx_gemm_pipe_kernel(const GemmParams p) {
     auto issue_tile_load = [&](int slot, int i, uint32_t koff) {
         dma_b128(dma_base + slot * kSlotBytes + i * (NW * 1024), goff[i], i < kWTileLoads ? w_rs : a_rs, koff);
     };
+    const uint32_t pf_sink = __builtin_amdgcn_readfirstlane(lds0 + kScaleBase + kScaleRingBytes + 256);
+    auto issue_prefetch = [&](int j, uint32_t koff) { dma_b32(pf_sink, pfoff[j], pf_rs, koff); };
     auto issue_scale_loads = [&](int slot, uint32_t soff) {          // one slab (three-slot kernel)
         dma_b32(sdma_base + slot * kScaleSlotBytes, sgoff_w, ws_rs, soff);
         dma_b32(sdma_base_a + slot * kScaleSlotBytes, sgoff_a, as_rs, soff);
@@ -333,7 +378,12 @@ __global__ __launch_bounds__(256) void mx_gemm_pipe_kernel(const GemmParams p) {
         const uint32_t k1 = clamp_slab(1);
 #pragma unroll
         for (int i = 0; i < kTileLoads; ++i) issue_tile_load(1, i, k1 * kSlabBytes);
-        asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(kTileLoads) : "memory");      // slab 0 and its scales have landed everywhere
+        if constexpr (kPf > 0) {
+            const uint32_t kp = clamp_slab(1 + kPfAhead) * kSlabBytes;
+            issue_prefetch(0, kp);
+            issue_prefetch(1, kp);
+        }
+        asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(kTileLoads + kPf) : "memory");      // slab 0 and its scales have landed everywhere
         static_for<0, NF>([&](auto ic) { read_frag(I0{}, I0{}, ic, f0lo, f0hi); });
         {
             const uint32_t off = scale_read_offset();
@@ -398,7 +448,8 @@ __global__ __launch_bounds__(256) void mx_gemm_pipe_kernel(const GemmParams p) {
     // MFMAs of a step; after MFMA kB1 the last of them has had time to land; kEarly tile loads of slab s+2
     // are issued already in step 0, behind the first barrier.
     // q = slab of the load stream within its tile (kNoSlab: nothing new to request, re-request slab koff)
-    auto slab_body2 = [&](auto slot_c, uint32_t koff, uint32_t q) {
+    // kpf = byte offset of the slab to prefetch (two-by-two persistent kernels)
+    auto slab_body2 = [&](auto slot_c, uint32_t koff, uint32_t q, uint32_t kpf) {
         constexpr int slot = decltype(slot_c)::value;
         constexpr int kR = NF > 8 ? 3 : 2;
         constexpr int kB1 = (kReads + kR - 1) / kR;
@@ -425,7 +476,7 @@ __global__ __launch_bounds__(256) void mx_gemm_pipe_kernel(const GemmParams p) {
         pin_fragments(f0lo, f0hi);
         // own loads of slab s+1 are complete (only the kEarly loads just issued may be in flight); after the
         // barrier so are everyone's
-        asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(kEarly) : "memory");
+        asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(kEarly + kPf) : "memory");
         // ---- step 1 ----
         static_for<0, kM>([&](auto ic) {
             constexpr int i = decltype(ic)::value;
@@ -446,6 +497,9 @@ __global__ __launch_bounds__(256) void mx_gemm_pipe_kernel(const GemmParams p) {
                 asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
                 shift_scales(OtherT{});
             }
+            // behind every tile load and the scale block of this slab: the waits above count on that order
+            if constexpr (kPf > 0 && i == kB1 + kScaleMfmas) issue_prefetch(0, kpf);
+            if constexpr (kPf > 0 && i == kB1 + kScaleMfmas + 2) issue_prefetch(1, kpf);
         });
         pin_fragments(f1lo, f1hi);
         pin_scales(SlotT{});
@@ -532,8 +586,8 @@ __global__ __launch_bounds__(256) void mx_gemm_pipe_kernel(const GemmParams p) {
     } else if constexpr (!kPersistent) {
         for (uint32_t s = 0; s < nslab; s += 2) {      // the host only selects this kernel for a slab count that is a multiple of four
             const uint32_t q0 = s + 2, q1 = s + 3;
-            slab_body2(I0{}, clamp_slab(q0) * kSlabBytes, q0 < nslab ? q0 : kNoSlab);
-            slab_body2(I1{}, clamp_slab(q1) * kSlabBytes, q1 < nslab ? q1 : kNoSlab);
+            slab_body2(I0{}, clamp_slab(q0) * kSlabBytes, q0 < nslab ? q0 : kNoSlab, 0);
+            slab_body2(I1{}, clamp_slab(q1) * kSlabBytes, q1 < nslab ? q1 : kNoSlab, 0);
         }
         asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
         fence_accumulators();
@@ -566,8 +620,8 @@ __global__ __launch_bounds__(256) void mx_gemm_pipe_kernel(const GemmParams p) {
                     sq = 0;
                 }
             }
-            slab_body2(I0{}, clamp_slab(sq) * kSlabBytes, sq < nslab ? sq : kNoSlab);
-            slab_body2(I1{}, clamp_slab(sq + 1) * kSlabBytes, sq + 1 < nslab ? sq + 1 : kNoSlab);
+            slab_body2(I0{}, clamp_slab(sq) * kSlabBytes, sq < nslab ? sq : kNoSlab, clamp_slab(sq + kPfAhead) * kSlabBytes);
+            slab_body2(I1{}, clamp_slab(sq + 1) * kSlabBytes, sq + 1 < nslab ? sq + 1 : kNoSlab, clamp_slab(sq + 1 + kPfAhead) * kSlabBytes);
             sq += 2;
             sm += 2;
             if (sm == nslab) {

@@ -35,6 +35,10 @@ __device__ __forceinline__ void dma_b128_aimed(uint32_t voff, v4i rsrc, uint32_t
     soff = __builtin_amdgcn_readfirstlane(soff);
     asm volatile("buffer_load_dwordx4 %0, %1, %2 offen lds" ::"v"(voff), "s"(rsrc), "s"(soff) : "memory");
 }
+__device__ __forceinline__ void dma_b32_aimed(uint32_t voff, v4i rsrc, uint32_t soff) {
+    soff = __builtin_amdgcn_readfirstlane(soff);
+    asm volatile("buffer_load_dword %0, %1, %2 offen lds" ::"v"(voff), "s"(rsrc), "s"(soff) : "memory");
+}
 typedef int v2i __attribute__((ext_vector_type(2)));
 template <int OFF>
 __device__ __forceinline__ v2i lds_read_b64(uint32_t addr) {
@@ -82,6 +86,9 @@ __global__ __launch_bounds__(256) void mx_gemm_pipe_fp4_kernel(const GemmParams 
     constexpr int kTileLoads = kRows / (8 * NW);              // 16
     constexpr int kWTileLoads = TW / (8 * NW);
     static_assert(kM == 16 && NF + NF / 2 < kM, "schedule is written for 16 MFMAs per step");
+    // L2 prefetch of the persistent 2 x 2 kernels, as in mx_gemm_pipe_kernel: two loads per wavefront and slab
+    constexpr int kPfAhead = (pipe_is_persistent(2, EPI) && WW == 2 && WM == 2) ? CMX_PIPE_PREFETCH : 0;
+    constexpr int kPf = kPfAhead > 0 ? 2 : 0;
 
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t*)smem;
@@ -107,6 +114,8 @@ __global__ __launch_bounds__(256) void mx_gemm_pipe_fp4_kernel(const GemmParams 
     Tile tq;
     v4i w_rs, a_rs, ws_rs, as_rs;
     uint32_t goff[kTileLoads], sgoff_w, sgoff_a;
+    uint32_t pfoff[2] = {0, 0};                 // prefetch: wavefronts 0, 1 cover the weight rows, 2, 3 the activation rows
+    v4i pf_rs = {0, 0, 0, 0};
     auto make_rsrc = [](const uint8_t* q) -> v4i {
         const uint64_t v = reinterpret_cast<uint64_t>(q);
         v4i r;
@@ -143,6 +152,25 @@ __global__ __launch_bounds__(256) void mx_gemm_pipe_fp4_kernel(const GemmParams 
         }
         sgoff_w = wrow_of(64 * wave + lane) * p.ld_ws;
         sgoff_a = arow_of(64 * wave + lane) * p.ld_as;
+        if constexpr (kPf > 0) {
+            // each workgroup prefetches its share of the panels it has in common with its neighbours on the XCD
+            const uint32_t band = p.row_off != nullptr ? 8u : 4u;
+            const uint32_t mtg = p.row_off != nullptr ? (uint32_t)p.tile_pref[g + 1] - (uint32_t)p.tile_pref[g] : m_tiles_all;
+            const uint32_t mt = tq.mt, b0 = mt / band * band;
+            const uint32_t band_rows = __builtin_amdgcn_readfirstlane(mtg - b0 < band ? mtg - b0 : band);
+            uint32_t nsh_a = 32u / band_rows;
+            nsh_a = __builtin_amdgcn_readfirstlane(nsh_a < p.w_tiles ? nsh_a : p.w_tiles);
+            const uint32_t mod = wave < 2 ? band_rows : nsh_a;
+            const uint32_t sel = __builtin_amdgcn_readfirstlane(wave < 2 ? mt - b0 : wt % nsh_a);
+            const uint32_t last = __builtin_amdgcn_readfirstlane(sel + mod * ((255u - sel) / mod));
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+                uint32_t r = sel + mod * ((2 * (wave & 1u) + j) * 64 + lane);
+                r = (r < 256u && mod >= 4u) ? r : last;      // a panel with fewer than four sharers is left to its own tile loads
+                pfoff[j] = wave < 2 ? mul_lo_u32(wrow_of(r), p.ldw) : mul_lo_u32(arow_of(r), p.lda);
+            }
+            pf_rs = wave < 2 ? w_rs : a_rs;
+        }
     };
     aim_loads_at(tile_id, 0);
     Tile tc = tq;                               // tile of the MFMA stream / epilogue
@@ -158,6 +186,7 @@ __global__ __launch_bounds__(256) void mx_gemm_pipe_fp4_kernel(const GemmParams 
     // the same in two halves, with an MFMA between them
     auto aim_tile_load = [&](int slot, int i) { dma_aim(dma_base + slot * kSlotBytes + i * (NW * 1024)); };
     auto fire_tile_load = [&](int i, uint32_t slab) { dma_b128_aimed(goff[i], i < kWTileLoads ? w_rs : a_rs, slab * kSlabBytes); };
+    const uint32_t pf_sink = __builtin_amdgcn_readfirstlane(lds0 + kScaleBase + 2 * kScaleSlotBytes + 256);
     // block `blk` of the load stream's tile (the scales of its slabs 2 blk and 2 blk + 1) into the next ring position
     const uint32_t nblk = nslab / 2;
     uint32_t blocks_issued = 0;          // running count over all tiles of this workgroup: ring position = count & 1
@@ -260,7 +289,12 @@ __global__ __launch_bounds__(256) void mx_gemm_pipe_fp4_kernel(const GemmParams 
 #pragma unroll
         for (int i = 0; i < kTileLoads; ++i) issue_tile_load(1, i, k1);
     }
-    asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(kTileLoads) : "memory");      // slab 0 and its scales have landed everywhere
+    if constexpr (kPf > 0) {
+        const uint32_t kp = clamp_slab(1 + kPfAhead) * kSlabBytes;
+        dma_b32(pf_sink, pfoff[0], pf_rs, kp);
+        dma_b32(pf_sink, pfoff[1], pf_rs, kp);
+    }
+    asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(kTileLoads + kPf) : "memory");      // slab 0 and its scales have landed everywhere
     // step 0 of the slab in slot 0 and its scales into fragment set a / scale set 0
     auto read_first_step = [&]() {
         static_for<0, NF>([&](auto ic) { read_piece(I0{}, I0{}, ic, fa); });
@@ -288,7 +322,8 @@ __global__ __launch_bounds__(256) void mx_gemm_pipe_fp4_kernel(const GemmParams 
     constexpr int kEarly = kM - kB1 - 1;        // tile loads of slab s+2 issued in step 2 (6)
     constexpr uint32_t kNoSlab = 0xFFFFFFFFu;
     // q = slab of the load stream within its tile (kNoSlab: nothing new to request, slab q2 is requested again)
-    auto slab_body = [&](auto slot_c, uint32_t q2, uint32_t q) {
+    // qpf = slab to prefetch (persistent 2 x 2 kernels)
+    auto slab_body = [&](auto slot_c, uint32_t q2, uint32_t q, uint32_t qpf) {
         constexpr int slot = decltype(slot_c)::value;
         using SlotT = std::integral_constant<int, slot>;
         using OtherT = std::integral_constant<int, slot ^ 1>;
@@ -335,17 +370,21 @@ __global__ __launch_bounds__(256) void mx_gemm_pipe_fp4_kernel(const GemmParams 
         pin_fragments(fa);
         // own loads of slab s+1 are complete (only the kEarly loads just issued may be in flight); after the
         // barrier so are everyone's
-        asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(kEarly) : "memory");
+        asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(kEarly + kPf) : "memory");
         // ---- step 3: the other loads, the first fragments of the next slab ----
         static_for<0, kM>([&](auto ic) {
             constexpr int i = decltype(ic)::value;
             if constexpr (i + kEarly < kTileLoads) aim_tile_load(slot, i + kEarly);
+            // the prefetch loads go behind every tile load and the scale block of this slab: the waits count on that order
+            if constexpr (kPf > 0 && (i == kTileLoads - kEarly + 2 || i == kTileLoads - kEarly + 4)) dma_aim(pf_sink);
             step_mfma(I3{}, ic, fb, SlotT{});
             if constexpr (i < NF) read_piece(OtherT{}, I0{}, ic, fa);
             if constexpr (i + kEarly < kTileLoads) fire_tile_load(i + kEarly, q2);
             if constexpr (i + kEarly == kTileLoads) {
                 if (q != kNoSlab && scale_block_due(q)) issue_scale_block(scale_block_of(q));
             }
+            if constexpr (kPf > 0 && i == kTileLoads - kEarly + 2) dma_b32_aimed(pfoff[0], pf_rs, qpf * kSlabBytes);
+            if constexpr (kPf > 0 && i == kTileLoads - kEarly + 4) dma_b32_aimed(pfoff[1], pf_rs, qpf * kSlabBytes);
         });
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");      // fragment set a of the next slab
         pin_fragments(fb);
@@ -363,8 +402,8 @@ __global__ __launch_bounds__(256) void mx_gemm_pipe_fp4_kernel(const GemmParams 
     if constexpr (!kPersistent) {
         for (uint32_t s = 0; s < nslab; s += 2) {      // the host only selects this kernel for an even slab count
             const uint32_t q0 = s + 2, q1 = s + 3;
-            slab_body(I0{}, clamp_slab(q0), q0 < nslab ? q0 : kNoSlab);
-            slab_body(I1{}, clamp_slab(q1), q1 < nslab ? q1 : kNoSlab);
+            slab_body(I0{}, clamp_slab(q0), q0 < nslab ? q0 : kNoSlab, 0);
+            slab_body(I1{}, clamp_slab(q1), q1 < nslab ? q1 : kNoSlab, 0);
         }
         asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
         fence_accumulators();
@@ -393,8 +432,8 @@ __global__ __launch_bounds__(256) void mx_gemm_pipe_fp4_kernel(const GemmParams 
                     sq = 0;
                 }
             }
-            slab_body(I0{}, clamp_slab(sq), sq < nslab ? sq : kNoSlab);
-            slab_body(I1{}, clamp_slab(sq + 1), sq + 1 < nslab ? sq + 1 : kNoSlab);
+            slab_body(I0{}, clamp_slab(sq), sq < nslab ? sq : kNoSlab, clamp_slab(sq + kPfAhead));
+            slab_body(I1{}, clamp_slab(sq + 1), sq + 1 < nslab ? sq + 1 : kNoSlab, clamp_slab(sq + 1 + kPfAhead));
             sq += 2;
             sm += 2;
             if (sm == nslab) {
