@@ -65,10 +65,14 @@ def main() -> int:
 
     def hip_time(fn, steps=K_STEPS, warm=max(WARM, 25)):
         """Average duration (s) of fn() over `steps` launches, HIP events on the launch stream (the extras: at least 25
-        untimed launches first, past the power-management ramp that follows a change of load)."""
-        for _ in range(warm):
-            fn()
-        torch.cuda.synchronize()
+        untimed launches and 30 ms first, past the power-management ramp that follows a change of load)."""
+        t_warm = time.perf_counter()
+        while True:
+            for _ in range(warm):
+                fn()
+            torch.cuda.synchronize()
+            if time.perf_counter() - t_warm >= 0.03:      # the clock needs about 20 ms of a new load to settle, however many launches that is
+                break
         e0 = torch.cuda.Event(enable_timing=True)
         e1 = torch.cuda.Event(enable_timing=True)
         e0.record()

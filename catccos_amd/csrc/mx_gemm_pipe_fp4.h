@@ -166,7 +166,9 @@ __global__ __launch_bounds__(256) void mx_gemm_pipe_fp4_kernel(const GemmParams 
 #pragma unroll
             for (int j = 0; j < 2; ++j) {
                 uint32_t r = sel + mod * ((2 * (wave & 1u) + j) * 64 + lane);
-                r = (r < 256u && mod >= 4u) ? r : last;      // a panel with fewer than four sharers is left to its own tile loads
+                // a panel with fewer than four sharers is left to its own tile loads; so are dense problems, whose workgroups
+                // run in lock step (measured: 182.8 us without, 184.8 / 187.1 us with a prefetch 1 / 2 slabs ahead)
+                r = (r < 256u && mod >= 4u && p.row_off != nullptr) ? r : last;
                 pfoff[j] = wave < 2 ? mul_lo_u32(wrow_of(r), p.ldw) : mul_lo_u32(arow_of(r), p.lda);
             }
             pf_rs = wave < 2 ? w_rs : a_rs;
