@@ -394,8 +394,10 @@ __device__ __forceinline__ void epilogue(const GemmParams& p, const Tile& tc, v1
                     }
                 }
                 uint32_t amax = max(m & 0xFFFFu, m >> 16);
-                const uint32_t other = (uint32_t)__shfl_xor((int)amax, 32);
-                amax = amax > other ? amax : other;
+                // the other half of the block's columns sits in lane l ^ 32: swap the half-waves of two copies in the
+                // register file (no trip through the LDS crossbar, no lgkmcnt wait between the blocks)
+                const auto both = __builtin_amdgcn_permlane32_swap(amax, amax, false, false);
+                amax = max(both[0], both[1]);
                 const int e = block_exp_from_bf16_amax(amax, kEmaxE4M3);
                 if (!mvalid || ncol0 >= half) continue;
                 // clamp the magnitudes to 448 * 2^e on the bit patterns, divide by 2^e and cast in one instruction
