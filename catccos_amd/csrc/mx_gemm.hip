@@ -60,7 +60,7 @@ struct GemmParams {
     uint16_t* act_bf16;
     const int32_t* row_off;     // [groups+1] (grouped) or null (dense)
     const int32_t* tile_pref;   // [groups+1] prefix of m-tiles (grouped) or null
-    int32_t* tile_ctr;          // [8] per-XCD tile counters, zeroed before the launch (persistent grouped kernels) or null
+    int32_t* tile_ctr;          // [8] per-XCD tile counters, zeroed before the launch (persistent grouped 4 x 1 kernels) or null
     uint32_t lda, ld_as, ldw, ld_ws, ldc, ld_act, ld_acts;
     uint32_t m, n, kbytes, kblocks;   // kblocks = K/32
     uint32_t groups, w_tiles;
@@ -136,11 +136,19 @@ struct Tile {
     uint32_t g, mt, wt, row0, rows_valid;
 };
 
+// The group tables (row offsets, m-tile prefix) are written by gmm_prepare_kernel before the matmul kernel starts and
+// never change under it: reading them through the constant address space lets a wavefront-uniform lookup use scalar
+// loads, which wait on lgkmcnt and so do not drain the LDS-DMA loads a persistent kernel has in flight (a vector load
+// would: its s_waitcnt vmcnt covers everything issued before it).
+__device__ __forceinline__ int32_t table_at(const int32_t* t, uint32_t i) {
+    return ((const __attribute__((address_space(4))) int32_t*)t)[i];
+}
+
 // Tiles are numbered linearly: within a group m-tiles run fastest so that neighbours share a weight panel;
 // dense problems walk bands of four m-tiles across a run of weight tiles.
 template <int TM>
 __device__ __forceinline__ uint32_t count_m_tiles(const GemmParams& p) {
-    return p.row_off != nullptr ? (uint32_t)p.tile_pref[p.groups] : (p.m + TM - 1) / TM;
+    return p.row_off != nullptr ? (uint32_t)table_at(p.tile_pref, p.groups) : (p.m + TM - 1) / TM;
 }
 
 // Tile L of an XCD-aware order: linear ids congruent mod 8 run on one XCD; each XCD gets a contiguous run.
@@ -161,19 +169,19 @@ __device__ __forceinline__ void decode_tile(const GemmParams& p, uint32_t m_tile
         const uint32_t G = p.groups;
         uint32_t lo = g_from, hi = G;
         const uint32_t i2 = lo + 2 < G ? lo + 2 : G, i3 = lo + 3 < G ? lo + 3 : G;
-        const uint32_t t1 = (uint32_t)p.tile_pref[lo + 1] * p.w_tiles, t2 = (uint32_t)p.tile_pref[i2] * p.w_tiles,
-                       t3 = (uint32_t)p.tile_pref[i3] * p.w_tiles;
+        const uint32_t t1 = (uint32_t)table_at(p.tile_pref, lo + 1) * p.w_tiles, t2 = (uint32_t)table_at(p.tile_pref, i2) * p.w_tiles,
+                       t3 = (uint32_t)table_at(p.tile_pref, i3) * p.w_tiles;
         if (t1 > L) hi = lo + 1;
         else if (t2 > L) { lo += 1; hi = lo + 1; }
         else if (t3 > L) { lo += 2; hi = lo + 1; }
         else lo += 3;
         while (hi - lo > 1) {
             const uint32_t mid = (lo + hi) >> 1;
-            if ((uint32_t)p.tile_pref[mid] * p.w_tiles <= L) lo = mid; else hi = mid;
+            if ((uint32_t)table_at(p.tile_pref, mid) * p.w_tiles <= L) lo = mid; else hi = mid;
         }
         t.g = lo;
-        const uint32_t tp = (uint32_t)p.tile_pref[lo];
-        const uint32_t mtg = (uint32_t)p.tile_pref[lo + 1] - tp;
+        const uint32_t tp = (uint32_t)table_at(p.tile_pref, lo);
+        const uint32_t mtg = (uint32_t)table_at(p.tile_pref, lo + 1) - tp;
         // bands of 8 m-tiles share a run of weight tiles (m fastest inside a band): the 32 tiles that an XCD
         // works on at a time then touch 8 + 4 operand panels instead of mtg + 32/mtg
         const uint32_t local = L - tp * p.w_tiles;
@@ -183,7 +191,7 @@ __device__ __forceinline__ void decode_tile(const GemmParams& p, uint32_t m_tile
         const uint32_t band_rows = (mtg - b * band) < band ? (mtg - b * band) : band;
         t.mt = b * band + within % band_rows;
         t.wt = within / band_rows;
-        const uint32_t r_begin = (uint32_t)p.row_off[lo], r_end = (uint32_t)p.row_off[lo + 1];
+        const uint32_t r_begin = (uint32_t)table_at(p.row_off, lo), r_end = (uint32_t)table_at(p.row_off, lo + 1);
         t.row0 = r_begin + t.mt * TM;
         t.rows_valid = r_end - t.row0 < (uint32_t)TM ? r_end - t.row0 : (uint32_t)TM;
     } else {
@@ -1271,7 +1279,10 @@ int gmm_common(GemmParams& p, const int32_t* group_sizes, uint32_t groups, uint3
     CMX_LAUNCH_CHECK();
     p.row_off = row_off;
     p.tile_pref = tile_pref;
-    p.tile_ctr = tile_ctr;
+    // The persistent kernels draw their next tile from a per-XCD counter when tiles differ in cost (4 x 1 wavefronts skip
+    // the MFMAs of absent rows).  With 2 x 2 wavefronts every tile costs the same, so those kernels walk their XCD's run in
+    // fixed strides instead: no atomic whose result has to be waited for with everything else in flight.
+    p.tile_ctr = t.waves == 4 ? nullptr : tile_ctr;
     p.groups = groups;
     p.w_tiles = swiglu ? ceil_div(p.n / 2, t.tw / 2) : ceil_div(p.n, t.tw);
     const uint32_t max_m_tiles = m_total / t.tm + groups;

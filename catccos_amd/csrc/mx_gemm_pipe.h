@@ -244,7 +244,7 @@ __global__ __launch_bounds__(256) void mx_gemm_pipe_kernel(const GemmParams p) {
             // activation panel with the neighbouring weight tiles.  Each prefetches only its share of a panel's rows
             // (row = position in the sharing set, modulo its size); the lanes left over repeat the last such row.
             const uint32_t band = p.row_off != nullptr ? 8u : 4u;
-            const uint32_t mtg = p.row_off != nullptr ? (uint32_t)p.tile_pref[g + 1] - (uint32_t)p.tile_pref[g] : m_tiles_all;
+            const uint32_t mtg = p.row_off != nullptr ? (uint32_t)table_at(p.tile_pref, g + 1) - (uint32_t)table_at(p.tile_pref, g) : m_tiles_all;
             const uint32_t mt = tq.mt, b0 = mt / band * band;
             const uint32_t band_rows = __builtin_amdgcn_readfirstlane(mtg - b0 < band ? mtg - b0 : band);
             uint32_t nsh_a = 32u / band_rows;
@@ -600,7 +600,7 @@ __global__ __launch_bounds__(256) void mx_gemm_pipe_kernel(const GemmParams p) {
         // re-requesting the last slab when there is none), so the loads and the fragment reads run on through
         // the tile boundary and only the epilogue and the clearing of the accumulators interrupt the MFMAs.
         // One loop holds every case so that the register assignment of the scheduled part never changes.
-        // Next tile: with a counter array (grouped problems, whose tiles differ in cost) the workgroups of an
+        // Next tile: with a counter array (grouped problems in the 4 x 1 layout, whose tiles differ in cost) the workgroups of an
         // XCD draw from that XCD's run in order; without one the walk is strided.
         uint32_t sm = 0;             // slab of the MFMA stream within its tile
         uint32_t sq = 2;             // slab of the load stream within its tile

@@ -155,7 +155,7 @@ __global__ __launch_bounds__(256) void mx_gemm_pipe_fp4_kernel(const GemmParams 
         if constexpr (kPf > 0) {
             // each workgroup prefetches its share of the panels it has in common with its neighbours on the XCD
             const uint32_t band = p.row_off != nullptr ? 8u : 4u;
-            const uint32_t mtg = p.row_off != nullptr ? (uint32_t)p.tile_pref[g + 1] - (uint32_t)p.tile_pref[g] : m_tiles_all;
+            const uint32_t mtg = p.row_off != nullptr ? (uint32_t)table_at(p.tile_pref, g + 1) - (uint32_t)table_at(p.tile_pref, g) : m_tiles_all;
             const uint32_t mt = tq.mt, b0 = mt / band * band;
             const uint32_t band_rows = __builtin_amdgcn_readfirstlane(mtg - b0 < band ? mtg - b0 : band);
             uint32_t nsh_a = 32u / band_rows;
