@@ -117,17 +117,18 @@ __device__ __forceinline__ v8i join8(const v4i& lo, const v4i& hi) {
 //           rate, sets the pace.
 __host__ __device__ constexpr bool pipe_is_persistent(int nslot, int epi) { return nslot == 2 && epi != kEpiStore; }
 
-// L2 prefetch distance in slabs for the persistent 2 x 2 kernels (0: none).  While the load stream requests slab q,
-// the workgroup also touches one dword of every 128-byte line of slab q + distance -- of its share of the rows: the
-// workgroups that run side by side on an XCD share operand panels, and each takes the rows congruent to its position
-// in the sharing set, so every line is asked for once per XCD, one to two slab times before the LDS-DMA loads of
-// all sharers want it.  The loads have no register destination (they land in a 256-byte LDS sink nobody reads), and
-// they are issued behind the tile loads of their slab, so every wait in the schedule simply lets two more loads stay
-// in flight.  Loads return in order, so a prefetch must be back within about one and a half slab times or it holds
-// up the tile loads behind it: distances 1 and 2 gain 4-5 % on the Zipf-routed 16-expert problem, 4 gains 2 %, 10
-// nothing (the further ahead, the more often the line comes all the way from HBM).  Prefetching every line of the
-// tile from every workgroup instead (512 instead of 96 lines per slab) costs 20 %: the price is per distinct line,
-// which is why a panel that fewer than four workgroups share is not prefetched at all.
+// L2 prefetch distance in slabs for the persistent 2 x 2 kernels (0: none).  The workgroups that run side by side on
+// an XCD share operand panels, and without help the one that is furthest ahead pays the HBM latency of every shared
+// line for all of them.  While the load stream requests slab q, the workgroup therefore also touches one dword of
+// every 128-byte line of slab q + distance -- of its share of the weight panel's rows: the m-tiles of a band share the
+// panel, and each takes the rows congruent to its position in the band, so every line is asked for once per XCD, one
+// to two slab times before the LDS-DMA loads of all sharers want it.  The loads have no register destination (they
+// land in a 256-byte LDS sink nobody reads), and they are issued behind the tile loads of their slab, so every wait in
+// the schedule simply lets two more loads stay in flight.  Loads return in order, so a prefetch must be back within
+// about one and a half slab times or it holds up the tile loads behind it: distances 1 to 3 gain 4-5 % on the
+// Zipf-routed 16-expert problem, 4 gains less, 10 nothing (the further ahead, the more often the line comes all the
+// way from HBM).  The price is per distinct line: prefetching every line of the tile from every workgroup (512 lines per
+// slab instead of 32) costs 20 %, and the activation panels, which only four workgroups share, lose more than they gain.
 #ifndef CMX_PIPE_PREFETCH
 #define CMX_PIPE_PREFETCH 2
 #endif
@@ -187,8 +188,7 @@ __global__ __launch_bounds__(256) void mx_gemm_pipe_kernel(const GemmParams p) {
     Tile tq;                                    // tile of the load stream
     v4i w_rs, a_rs, ws_rs, as_rs;
     uint32_t goff[kTileLoads], sgoff_w, sgoff_a;
-    uint32_t pfoff[2] = {0, 0};                 // prefetch: wavefronts 0, 1 cover the weight rows, 2, 3 the activation rows
-    v4i pf_rs = {0, 0, 0, 0};
+    uint32_t pfoff[2] = {0, 0};                 // prefetch: weight rows of this workgroup's share (wavefront 0; the others repeat one row)
     const uint32_t sa_blk = wave % (TM / 64);
     auto make_rsrc = [](const uint8_t* q) -> v4i {
         const uint64_t v = reinterpret_cast<uint64_t>(q);
@@ -240,27 +240,26 @@ __global__ __launch_bounds__(256) void mx_gemm_pipe_kernel(const GemmParams p) {
         if constexpr (kPf > 0) {
             static_assert(kPf == 0 || (TW == 256 && TM == 256), "the prefetch split assumes 256 + 256 rows");
             // The workgroups that run side by side on an XCD share operand panels (tile order: bands of m-tiles, m
-            // fastest, across a run of weight tiles): the weight panel with the other m-tiles of the band, the
-            // activation panel with the neighbouring weight tiles.  Each prefetches only its share of a panel's rows
-            // (row = position in the sharing set, modulo its size); the lanes left over repeat the last such row.
+            // fastest, across a run of weight tiles): the weight panel with the other m-tiles of the band.  Each
+            // prefetches only its share of the panel's rows (row = position in the band, modulo the band's height);
+            // the lanes left over repeat the last such row.
             const uint32_t band = p.row_off != nullptr ? 8u : 4u;
             const uint32_t mtg = p.row_off != nullptr ? (uint32_t)table_at(p.tile_pref, g + 1) - (uint32_t)table_at(p.tile_pref, g) : m_tiles_all;
             const uint32_t mt = tq.mt, b0 = mt / band * band;
-            const uint32_t band_rows = __builtin_amdgcn_readfirstlane(mtg - b0 < band ? mtg - b0 : band);
-            uint32_t nsh_a = 32u / band_rows;
-            nsh_a = __builtin_amdgcn_readfirstlane(nsh_a < p.w_tiles ? nsh_a : p.w_tiles);
-            const uint32_t mod = wave < 2 ? band_rows : nsh_a;
-            const uint32_t sel = __builtin_amdgcn_readfirstlane(wave < 2 ? mt - b0 : wt % nsh_a);
+            const uint32_t mod = __builtin_amdgcn_readfirstlane(mtg - b0 < band ? mtg - b0 : band);      // m-tiles that share the weight panel
+            const uint32_t sel = __builtin_amdgcn_readfirstlane(mt - b0);
             const uint32_t last = __builtin_amdgcn_readfirstlane(sel + mod * ((255u - sel) / mod));
 #pragma unroll
             for (int j = 0; j < 2; ++j) {
-                uint32_t r = sel + mod * ((2 * (wave & 1u) + j) * 64 + lane);
-                // a panel with fewer than four sharers is left to its own tile loads; so are dense problems, whose workgroups
-                // run in lock step (measured: 182.8 us without, 184.8 / 187.1 us with a prefetch 1 / 2 slabs ahead)
-                r = (r < 256u && mod >= 4u && p.row_off != nullptr) ? r : last;
-                pfoff[j] = wave < 2 ? mul_lo_u32(wrow_of(r), p.ldw) : mul_lo_u32(arow_of(r), p.lda);
+                // Weight panels only, and only when at least three m-tiles of the band share one: on the 16-expert problem
+                // the weight panels (up to eight sharers) gain 4.3 % alone, the activation panels (four weight tiles side
+                // by side) lose 1.7 % alone, both together gain 3.6 %; thresholds of 3 / 5 / 6 / 8 sharers for the weight
+                // panels: 855.6 / 859.4 / 861.1 / 869.3 us.  Dense problems, whose workgroups run in lock step, lose 1-2 %.
+                // At most 86 rows: the two loads of wavefront 0 cover them, every other lane repeats the last one.
+                uint32_t r = sel + mod * (j * 64 + lane);
+                r = (r < 256u && wave == 0 && mod >= 3u && p.row_off != nullptr) ? r : last;
+                pfoff[j] = mul_lo_u32(wrow_of(r), p.ldw);
             }
-            pf_rs = wave < 2 ? w_rs : a_rs;
         }
     };
     aim_loads_at(tile_id, 0);
@@ -277,7 +276,7 @@ __global__ __launch_bounds__(256) void mx_gemm_pipe_kernel(const GemmParams p) {
         dma_b128(dma_base + slot * kSlotBytes + i * (NW * 1024), goff[i], i < kWTileLoads ? w_rs : a_rs, koff);
     };
     const uint32_t pf_sink = __builtin_amdgcn_readfirstlane(lds0 + kScaleBase + kScaleRingBytes + 256);
-    auto issue_prefetch = [&](int j, uint32_t koff) { dma_b32(pf_sink, pfoff[j], pf_rs, koff); };
+    auto issue_prefetch = [&](int j, uint32_t koff) { dma_b32(pf_sink, pfoff[j], w_rs, koff); };
     auto issue_scale_loads = [&](int slot, uint32_t soff) {          // one slab (three-slot kernel)
         dma_b32(sdma_base + slot * kScaleSlotBytes, sgoff_w, ws_rs, soff);
         dma_b32(sdma_base_a + slot * kScaleSlotBytes, sgoff_a, as_rs, soff);

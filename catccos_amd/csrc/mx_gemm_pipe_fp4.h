@@ -114,8 +114,7 @@ __global__ __launch_bounds__(256) void mx_gemm_pipe_fp4_kernel(const GemmParams 
     Tile tq;
     v4i w_rs, a_rs, ws_rs, as_rs;
     uint32_t goff[kTileLoads], sgoff_w, sgoff_a;
-    uint32_t pfoff[2] = {0, 0};                 // prefetch: wavefronts 0, 1 cover the weight rows, 2, 3 the activation rows
-    v4i pf_rs = {0, 0, 0, 0};
+    uint32_t pfoff[2] = {0, 0};                 // prefetch: weight rows of this workgroup's share (wavefront 0; the others repeat one row)
     auto make_rsrc = [](const uint8_t* q) -> v4i {
         const uint64_t v = reinterpret_cast<uint64_t>(q);
         v4i r;
@@ -153,25 +152,24 @@ __global__ __launch_bounds__(256) void mx_gemm_pipe_fp4_kernel(const GemmParams 
         sgoff_w = wrow_of(64 * wave + lane) * p.ld_ws;
         sgoff_a = arow_of(64 * wave + lane) * p.ld_as;
         if constexpr (kPf > 0) {
-            // each workgroup prefetches its share of the panels it has in common with its neighbours on the XCD
+            // each workgroup prefetches its share of the weight panel it has in common with the other m-tiles of its band
             const uint32_t band = p.row_off != nullptr ? 8u : 4u;
             const uint32_t mtg = p.row_off != nullptr ? (uint32_t)table_at(p.tile_pref, g + 1) - (uint32_t)table_at(p.tile_pref, g) : m_tiles_all;
             const uint32_t mt = tq.mt, b0 = mt / band * band;
-            const uint32_t band_rows = __builtin_amdgcn_readfirstlane(mtg - b0 < band ? mtg - b0 : band);
-            uint32_t nsh_a = 32u / band_rows;
-            nsh_a = __builtin_amdgcn_readfirstlane(nsh_a < p.w_tiles ? nsh_a : p.w_tiles);
-            const uint32_t mod = wave < 2 ? band_rows : nsh_a;
-            const uint32_t sel = __builtin_amdgcn_readfirstlane(wave < 2 ? mt - b0 : wt % nsh_a);
+            const uint32_t mod = __builtin_amdgcn_readfirstlane(mtg - b0 < band ? mtg - b0 : band);      // m-tiles that share the weight panel
+            const uint32_t sel = __builtin_amdgcn_readfirstlane(mt - b0);
             const uint32_t last = __builtin_amdgcn_readfirstlane(sel + mod * ((255u - sel) / mod));
 #pragma unroll
             for (int j = 0; j < 2; ++j) {
-                uint32_t r = sel + mod * ((2 * (wave & 1u) + j) * 64 + lane);
-                // a panel with fewer than four sharers is left to its own tile loads; so are dense problems, whose workgroups
-                // run in lock step (measured: 182.8 us without, 184.8 / 187.1 us with a prefetch 1 / 2 slabs ahead)
-                r = (r < 256u && mod >= 4u && p.row_off != nullptr) ? r : last;
-                pfoff[j] = wave < 2 ? mul_lo_u32(wrow_of(r), p.ldw) : mul_lo_u32(arow_of(r), p.lda);
+                // Weight panels only, and only when at least three m-tiles of the band share one: on the 16-expert problem
+                // the weight panels (up to eight sharers) gain 4.3 % alone, the activation panels (four weight tiles side
+                // by side) lose 1.7 % alone, both together gain 3.6 %; thresholds of 3 / 5 / 6 / 8 sharers for the weight
+                // panels: 855.6 / 859.4 / 861.1 / 869.3 us.  Dense problems, whose workgroups run in lock step, lose 1-2 %.
+                // At most 86 rows: the two loads of wavefront 0 cover them, every other lane repeats the last one.
+                uint32_t r = sel + mod * (j * 64 + lane);
+                r = (r < 256u && wave == 0 && mod >= 3u && p.row_off != nullptr) ? r : last;
+                pfoff[j] = mul_lo_u32(wrow_of(r), p.ldw);
             }
-            pf_rs = wave < 2 ? w_rs : a_rs;
         }
     };
     aim_loads_at(tile_id, 0);
@@ -293,8 +291,8 @@ __global__ __launch_bounds__(256) void mx_gemm_pipe_fp4_kernel(const GemmParams 
     }
     if constexpr (kPf > 0) {
         const uint32_t kp = clamp_slab(1 + kPfAhead) * kSlabBytes;
-        dma_b32(pf_sink, pfoff[0], pf_rs, kp);
-        dma_b32(pf_sink, pfoff[1], pf_rs, kp);
+        dma_b32(pf_sink, pfoff[0], w_rs, kp);
+        dma_b32(pf_sink, pfoff[1], w_rs, kp);
     }
     asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(kTileLoads + kPf) : "memory");      // slab 0 and its scales have landed everywhere
     // step 0 of the slab in slot 0 and its scales into fragment set a / scale set 0
@@ -385,8 +383,8 @@ __global__ __launch_bounds__(256) void mx_gemm_pipe_fp4_kernel(const GemmParams 
             if constexpr (i + kEarly == kTileLoads) {
                 if (q != kNoSlab && scale_block_due(q)) issue_scale_block(scale_block_of(q));
             }
-            if constexpr (kPf > 0 && i == kTileLoads - kEarly + 2) dma_b32_aimed(pfoff[0], pf_rs, qpf * kSlabBytes);
-            if constexpr (kPf > 0 && i == kTileLoads - kEarly + 4) dma_b32_aimed(pfoff[1], pf_rs, qpf * kSlabBytes);
+            if constexpr (kPf > 0 && i == kTileLoads - kEarly + 2) dma_b32_aimed(pfoff[0], w_rs, qpf * kSlabBytes);
+            if constexpr (kPf > 0 && i == kTileLoads - kEarly + 4) dma_b32_aimed(pfoff[1], w_rs, qpf * kSlabBytes);
         });
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");      // fragment set a of the next slab
         pin_fragments(fb);
