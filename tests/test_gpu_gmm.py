@@ -75,8 +75,9 @@ def test_gmm_many_ragged_groups_every_row(tile):
                                          ("E2M1", 512, 5), ("E2M1", 1536, 5)])
 def test_more_tiles_than_workgroups_every_row(fmt, k, waves):
     """Enough tiles (about 300 of 256 x 256) that the persistent kernels, one workgroup per CU, walk on to a second
-    tile: the load stream crosses the tile boundary, the next tile comes from the per-XCD counters, and every
-    row of every group must still come out right, with the rows past the groups untouched."""
+    tile: the load stream crosses the tile boundary, the next tile comes from the per-XCD counters (4 x 1 wavefronts) or
+    a fixed stride (2 x 2), and every row of every group must still come out right, with the rows past the groups
+    untouched."""
     from catccos_amd import ops, _lib
     hooks_lib().cmx_debug_force_tile(256, 256, waves)
     rng = np.random.default_rng(91)
@@ -121,6 +122,56 @@ def test_swiglu_requant_more_tiles_than_workgroups(waves):
     assert np.array_equal(host(scales), ws2) and np.array_equal(host(codes), wq2)
     codes_p, scales_p = ops.mx_gmm_swiglu_quant(dev(aq), dev(asc), dev(wq), dev(ws), dev(np.array(counts, dtype=np.int32)), k)[:2]
     assert torch.equal(codes_p, codes) and torch.equal(scales_p, scales)        # same without the bf16 output
+
+
+@pytest.mark.parametrize("fmt", ["E4M3", "E2M1"])
+def test_groups_of_many_m_tiles_every_row(fmt):
+    """Groups of 3 to 12 m-tiles (bands of eight m-tiles plus a rest of 1, 3, 4 or 6): the persistent 2 x 2 kernels prefetch
+    each workgroup's share of the weight panel that the m-tiles of a band have in common, rows congruent to the tile's
+    position in the band, and walk their XCD's tiles in fixed strides.  Every row of every group against the oracle."""
+    from catccos_amd import ops
+    rng = np.random.default_rng(93)
+    counts = [2304, 0, 2048, 1300, 768, 1, 3000, 2815, 513]
+    n, k = 512, 1024
+    m = sum(counts)
+    if fmt == "E2M1":
+        aq, asc = O.mx_quant(rng.uniform(-2, 2, (m, k)).astype(np.float32), "E2M1")
+        qs = [O.mx_quant(rng.uniform(-2, 2, (n, k)).astype(np.float32), "E2M1") for _ in counts]
+        pack = O.pack_fp4
+    else:
+        aq, asc = O.mx_quant(O.bf16_round(rng.standard_normal((m, k)).astype(np.float32)))
+        qs = [O.mx_quant(O.bf16_round(rng.standard_normal((n, k)).astype(np.float32))) for _ in counts]
+        pack = lambda x: x
+    wq, ws = np.stack([q for q, _ in qs]), np.stack([s_ for _, s_ in qs])
+    c = ops.mx_gmm(dev(pack(aq)), dev(asc), dev(pack(wq)), dev(ws), dev(np.array(counts, dtype=np.int32)), k, fmt, "bf16")
+    bad, worst = close_bf16(host(c), O.mx_gmm_f32(aq, asc, wq, ws, counts, fmt, fmt))
+    assert bad == 0, (bad, worst)
+
+
+def test_swiglu_requant_groups_of_many_m_tiles():
+    """The fused GMM1 epilogue on the same kind of groups: the 2 x 2 kernel (weight-panel prefetch, strided walk) and the
+    4 x 1 kernel (neither) give the same codes and scales, and both requantise their own bf16 values exactly."""
+    from catccos_amd import ops
+    rng = np.random.default_rng(94)
+    counts = [2304, 0, 2048, 1300, 768, 1, 3000, 2815, 513]
+    n, k = 1024, 1024
+    m = sum(counts)
+    aq, asc = O.mx_quant(O.bf16_round(rng.standard_normal((m, k)).astype(np.float32)))
+    wq, ws = _weights(rng, len(counts), n, k, std=0.06)
+    args = (dev(aq), dev(asc), dev(wq), dev(ws), dev(np.array(counts, dtype=np.int32)), k)
+    lib = hooks_lib()
+    outs = {}
+    for waves in (4, 5):
+        lib.cmx_debug_force_tile(256, 256, waves)
+        codes, scales, act = ops.mx_gmm_swiglu_quant(*args, want_bf16=True)
+        wq2, ws2 = O.mx_quant_bf16(host(act), "E4M3", "rne")
+        assert np.array_equal(host(scales), ws2) and np.array_equal(host(codes), wq2), waves
+        outs[waves] = ops.mx_gmm_swiglu_quant(*args)[:2]
+        assert torch.equal(outs[waves][0], codes) and torch.equal(outs[waves][1], scales), waves
+    assert torch.equal(outs[4][0], outs[5][0]) and torch.equal(outs[4][1], outs[5][1])
+    _, act_g, _, _ = O.gmm1_swiglu_quant(aq, asc, wq, ws, counts)
+    bad, worst = close_bf16(host(act), O.bf16_bits_to_f32(act_g), rtol=2e-2)
+    assert bad == 0, (bad, worst)
 
 
 @pytest.mark.parametrize("tile", [None, (256, 128, 5), (128, 128, 4)])
