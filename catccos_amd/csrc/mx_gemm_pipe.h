@@ -335,9 +335,14 @@ __global__ __launch_bounds__(256) void mx_gemm_pipe_kernel(const GemmParams p) {
     // weight fragment f sits f*32 rows (SwiGLU: the gate fragments, then their up partners 128 rows on) below the base
 #define CMX_PIPE_WOFF(f) ((epi_is_swiglu_quant(EPI) ? ((f) < FW / 2 ? (f) * 32 : TW / 2 + ((f) - FW / 2) * 32) : (f) * 32))
     // one 16-byte read: r = 2 * position in the read order + half (0: registers 0-3, 1: registers 4-7)
+    // Persistent 2 x 2 kernels read the step-1 fragments weights first: the weight rows of a slot are then free four MFMAs into
+    // step 0 and their loads (the ones that come from HBM) go out five MFMAs earlier than the slot as a whole would allow,
+    // while the activation fragments are still being read (0.7 % on the 16-expert problem; three or four reads per
+    // MFMA to free the rows earlier still: slower).
+    constexpr bool kWFirst = kPf > 0;
     auto read_half = [&](auto slot_c, auto step_c, auto r_c, v4i (&flo)[NF], v4i (&fhi)[NF]) {
         constexpr int slot = decltype(slot_c)::value, step = decltype(step_c)::value, r = decltype(r_c)::value;
-        constexpr int idx = pipe_read_order<FW, FM>(r / 2), half = r % 2;
+        constexpr int idx = (kWFirst && step == 1) ? r / 2 : pipe_read_order<FW, FM>(r / 2), half = r % 2;
         (void)wb, (void)ab;
         v4i& dst = half ? fhi[idx] : flo[idx];
         if constexpr (idx < FW) dst = lds_read_b128<CMX_PIPE_WOFF(idx) * kSlabBytes>(wb[slot][2 * step + half]);
@@ -470,20 +475,30 @@ __global__ __launch_bounds__(256) void mx_gemm_pipe_kernel(const GemmParams p) {
                 constexpr int r = i * kR + decltype(jc)::value;
                 if constexpr (r < kReads) read_half(SlotT{}, I1{}, std::integral_constant<int, r>{}, f1lo, f1hi);
             });
+            if constexpr (kWFirst) {
+                // the weight rows of slot `slot` have been read for the last time (fragments 0..FW-1, kR halves per MFMA):
+                // once everyone is here they can be refilled, while the activation rows are still being read
+                constexpr int kBw = (2 * FW + kR - 1) / kR - 1;
+                if constexpr (i == kBw) asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+                if constexpr (i > kBw && i - kBw - 1 < kWTileLoads) issue_tile_load(slot, i - kBw - 1, koff);
+                if constexpr (i == kB1) asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+            } else {
             // slot `slot` has been read for the last time: once everyone is here it can be refilled
             if constexpr (i == kB1) asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
             if constexpr (i > kB1) issue_tile_load(slot, i - kB1 - 1, koff);
+            }
         });
         pin_fragments(f0lo, f0hi);
         // own loads of slab s+1 are complete (only the kEarly loads just issued may be in flight); after the
         // barrier so are everyone's
-        asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(kEarly + kPf) : "memory");
+        constexpr int kEarlyN = kWFirst ? kWTileLoads : kEarly;
+        asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(kEarlyN + kPf) : "memory");
         // ---- step 1 ----
         static_for<0, kM>([&](auto ic) {
             constexpr int i = decltype(ic)::value;
             step_mfma(I2{}, ic, f1lo, f1hi, SlotT{});
-            if constexpr (i + kEarly < kTileLoads) issue_tile_load(slot, i + kEarly, koff);
-            if constexpr (i + kEarly == kTileLoads) {
+            if constexpr (i + kEarlyN < kTileLoads) issue_tile_load(slot, i + kEarlyN, koff);
+            if constexpr (i + kEarlyN == kTileLoads) {
                 if (q != kNoSlab && scale_block_due(q)) issue_scale_block(scale_block_of(q));
             }
             static_for<0, kR>([&](auto jc) {

@@ -233,7 +233,9 @@ __global__ __launch_bounds__(256) void mx_gemm_pipe_fp4_kernel(const GemmParams 
 #define CMX_PIPE_WOFF(f) ((epi_pairs_gate_up(EPI) ? ((f) < FW / 2 ? (f) * 32 : TW / 2 + ((f) - FW / 2) * 32) : (f) * 32))
     auto read_piece = [&](auto slot_c, auto step_c, auto pos_c, v4i (&f)[NF]) {
         constexpr int slot = decltype(slot_c)::value, step = decltype(step_c)::value;
-        constexpr int idx = pipe_read_order<FW, FM>(decltype(pos_c)::value);
+        // the last step's fragments of a slot are read weights first in the persistent 2 x 2 kernels, so that the weight rows
+        // are free (and their loads go out) while the activation fragments are still being read
+        constexpr int idx = (kPf > 0 && step == 3) ? decltype(pos_c)::value : pipe_read_order<FW, FM>(decltype(pos_c)::value);
         (void)wb, (void)ab;
         if constexpr (idx < FW) f[idx] = lds_read_b128<CMX_PIPE_WOFF(idx) * kSlabBytes>(wb[slot][step]);
         else f[idx] = lds_read_b128<(idx - FW) * 32 * kSlabBytes>(ab[slot][step]);
@@ -320,6 +322,8 @@ __global__ __launch_bounds__(256) void mx_gemm_pipe_fp4_kernel(const GemmParams 
 
     constexpr int kB1 = 9;                      // MFMA of step 2 after which the reads of step 3 have landed
     constexpr int kEarly = kM - kB1 - 1;        // tile loads of slab s+2 issued in step 2 (6)
+    constexpr bool kWFirst = kPf > 0;           // persistent 2 x 2 kernels: the eight weight loads go out early instead (see read_piece)
+    constexpr int kEarlyN = kWFirst ? kWTileLoads : kEarly;
     constexpr uint32_t kNoSlab = 0xFFFFFFFFu;
     // q = slab of the load stream within its tile (kNoSlab: nothing new to request, slab q2 is requested again)
     // qpf = slab to prefetch (persistent 2 x 2 kernels)
@@ -361,30 +365,40 @@ __global__ __launch_bounds__(256) void mx_gemm_pipe_fp4_kernel(const GemmParams 
         // ---- step 2: last reads of the slot, first loads of slab s+2 ----
         static_for<0, kM>([&](auto ic) {
             constexpr int i = decltype(ic)::value;
-            if constexpr (i > kB1) aim_tile_load(slot, i - kB1 - 1);
-            step_mfma(I2{}, ic, fa, SlotT{});
-            if constexpr (i < NF) read_piece(SlotT{}, I3{}, ic, fb);
-            if constexpr (i == kB1) asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
-            if constexpr (i > kB1) fire_tile_load(i - kB1 - 1, q2);
+            if constexpr (kWFirst) {
+                // weight fragments 0..FW-1 are read behind MFMAs 0..FW-1: behind MFMA FW the weight rows of the slot are free
+                if constexpr (i > FW && i - FW - 1 < kWTileLoads) aim_tile_load(slot, i - FW - 1);
+                step_mfma(I2{}, ic, fa, SlotT{});
+                if constexpr (i < NF) read_piece(SlotT{}, I3{}, ic, fb);
+                if constexpr (i == FW) asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+                if constexpr (i > FW && i - FW - 1 < kWTileLoads) fire_tile_load(i - FW - 1, q2);
+                if constexpr (i == kB1) asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+            } else {
+                if constexpr (i > kB1) aim_tile_load(slot, i - kB1 - 1);
+                step_mfma(I2{}, ic, fa, SlotT{});
+                if constexpr (i < NF) read_piece(SlotT{}, I3{}, ic, fb);
+                if constexpr (i == kB1) asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+                if constexpr (i > kB1) fire_tile_load(i - kB1 - 1, q2);
+            }
         });
         pin_fragments(fa);
-        // own loads of slab s+1 are complete (only the kEarly loads just issued may be in flight); after the
+        // own loads of slab s+1 are complete (only the early loads just issued may be in flight); after the
         // barrier so are everyone's
-        asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(kEarly + kPf) : "memory");
+        asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(kEarlyN + kPf) : "memory");
         // ---- step 3: the other loads, the first fragments of the next slab ----
         static_for<0, kM>([&](auto ic) {
             constexpr int i = decltype(ic)::value;
-            if constexpr (i + kEarly < kTileLoads) aim_tile_load(slot, i + kEarly);
+            if constexpr (i + kEarlyN < kTileLoads) aim_tile_load(slot, i + kEarlyN);
             // the prefetch loads go behind every tile load and the scale block of this slab: the waits count on that order
-            if constexpr (kPf > 0 && (i == kTileLoads - kEarly + 2 || i == kTileLoads - kEarly + 4)) dma_aim(pf_sink);
+            if constexpr (kPf > 0 && (i == kTileLoads - kEarlyN + 2 || i == kTileLoads - kEarlyN + 4)) dma_aim(pf_sink);
             step_mfma(I3{}, ic, fb, SlotT{});
             if constexpr (i < NF) read_piece(OtherT{}, I0{}, ic, fa);
-            if constexpr (i + kEarly < kTileLoads) fire_tile_load(i + kEarly, q2);
-            if constexpr (i + kEarly == kTileLoads) {
+            if constexpr (i + kEarlyN < kTileLoads) fire_tile_load(i + kEarlyN, q2);
+            if constexpr (i + kEarlyN == kTileLoads) {
                 if (q != kNoSlab && scale_block_due(q)) issue_scale_block(scale_block_of(q));
             }
-            if constexpr (kPf > 0 && i == kTileLoads - kEarly + 2) dma_b32_aimed(pfoff[0], w_rs, qpf * kSlabBytes);
-            if constexpr (kPf > 0 && i == kTileLoads - kEarly + 4) dma_b32_aimed(pfoff[1], w_rs, qpf * kSlabBytes);
+            if constexpr (kPf > 0 && i == kTileLoads - kEarlyN + 2) dma_b32_aimed(pfoff[0], w_rs, qpf * kSlabBytes);
+            if constexpr (kPf > 0 && i == kTileLoads - kEarlyN + 4) dma_b32_aimed(pfoff[1], w_rs, qpf * kSlabBytes);
         });
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");      // fragment set a of the next slab
         pin_fragments(fb);

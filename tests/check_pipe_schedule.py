@@ -36,23 +36,23 @@ HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
          f"-I{os.path.join(ROOT, 'include')}", f"-I{HERE}", "-S", "--cuda-device-only", "-Wno-unused-command-line-argument"]
 
-# (explicit instantiation, the schedule's own vmcnt waits inside the stream: 7 early tile loads, plus 2 prefetch loads in the
-# persistent 2 x 2 kernels)
+# (explicit instantiation, the schedule's own vmcnt waits inside the stream: the early tile loads -- 7 or 8 (6 for FP4); the
+# persistent 2 x 2 kernels send all 8 weight loads early -- plus 2 prefetch loads in the persistent 2 x 2 kernels)
 #   mx_gemm_pipe_kernel<FMT, EPI, TM, WW, WM, NSLOT>; EPI 0 store, 1 SwiGLU + requant, 2 lean bf16, 4 lean fp16, 5 = 1 + bf16 activations
 #   mx_gemm_pipe_fp4_kernel<EPI, WW, WM>
 KERNELS = [
-    ("mx_gemm_pipe_kernel<0, 1, 256, 2, 2, 2>", {9}),
+    ("mx_gemm_pipe_kernel<0, 1, 256, 2, 2, 2>", {10}),
     ("mx_gemm_pipe_kernel<0, 1, 256, 4, 1, 2>", {8}),
-    ("mx_gemm_pipe_kernel<0, 5, 256, 2, 2, 2>", {9}),          # SwiGLU + requant that also writes the bf16 activations
+    ("mx_gemm_pipe_kernel<0, 5, 256, 2, 2, 2>", {10}),          # SwiGLU + requant that also writes the bf16 activations
     ("mx_gemm_pipe_kernel<0, 5, 256, 4, 1, 2>", {8}),
-    ("mx_gemm_pipe_kernel<0, 2, 256, 2, 2, 2>", {9}),
-    ("mx_gemm_pipe_kernel<0, 4, 256, 2, 2, 2>", {9}),
+    ("mx_gemm_pipe_kernel<0, 2, 256, 2, 2, 2>", {10}),
+    ("mx_gemm_pipe_kernel<0, 4, 256, 2, 2, 2>", {10}),
     ("mx_gemm_pipe_kernel<0, 0, 256, 2, 2, 2>", {7}),
     ("mx_gemm_pipe_kernel<0, 0, 256, 4, 1, 2>", {8}),
     ("mx_gemm_pipe_kernel<0, 0, 128, 4, 1, 3>", {14}),
     ("mx_gemm_pipe_kernel<0, 1, 128, 4, 1, 3>", {14}),
-    ("mx_gemm_pipe_fp4_kernel<2, 2, 2>", {8}),
-    ("mx_gemm_pipe_fp4_kernel<4, 2, 2>", {8}),
+    ("mx_gemm_pipe_fp4_kernel<2, 2, 2>", {10}),
+    ("mx_gemm_pipe_fp4_kernel<4, 2, 2>", {10}),
     ("mx_gemm_pipe_fp4_kernel<2, 4, 1>", {6}),
     ("mx_gemm_pipe_fp4_kernel<4, 4, 1>", {6}),
     ("mx_gemm_pipe_fp4_kernel<0, 2, 2>", {6}),
