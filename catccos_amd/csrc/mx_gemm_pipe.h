@@ -335,11 +335,13 @@ __global__ __launch_bounds__(256) void mx_gemm_pipe_kernel(const GemmParams p) {
     // weight fragment f sits f*32 rows (SwiGLU: the gate fragments, then their up partners 128 rows on) below the base
 #define CMX_PIPE_WOFF(f) ((epi_is_swiglu_quant(EPI) ? ((f) < FW / 2 ? (f) * 32 : TW / 2 + ((f) - FW / 2) * 32) : (f) * 32))
     // one 16-byte read: r = 2 * position in the read order + half (0: registers 0-3, 1: registers 4-7)
-    // Persistent 2 x 2 kernels read the step-1 fragments weights first: the weight rows of a slot are then free four MFMAs into
-    // step 0 and their loads (the ones that come from HBM) go out five MFMAs earlier than the slot as a whole would allow,
-    // while the activation fragments are still being read (0.7 % on the 16-expert problem; three or four reads per
-    // MFMA to free the rows earlier still: slower).
-    constexpr bool kWFirst = kPf > 0;
+    // The two-slot grouped kernels (persistent 2 x 2, and 4 x 1) read the step-1 fragments weights first: the weight rows of a
+    // slot are then free a few MFMAs into step 0 (four with 2 x 2 wavefronts, two with 4 x 1, whose wavefronts hold only two
+    // weight fragments), a barrier says so, and the eight weight loads of slab s+2 -- the ones that come from HBM -- go out
+    // five to six MFMAs earlier than the slot as a whole would allow, while the activation fragments are still being read.
+    // 0.7 % on the 16-expert problem (2 x 2), 3.2 % on GMM1 of the 256-expert FFN (4 x 1, private weight panels streamed
+    // from HBM).  Three or four reads per MFMA to free the rows earlier still: slower.
+    constexpr bool kWFirst = kPf > 0 || (kSkip && NSLOT == 2);
     auto read_half = [&](auto slot_c, auto step_c, auto r_c, v4i (&flo)[NF], v4i (&fhi)[NF]) {
         constexpr int slot = decltype(slot_c)::value, step = decltype(step_c)::value, r = decltype(r_c)::value;
         constexpr int idx = (kWFirst && step == 1) ? r / 2 : pipe_read_order<FW, FM>(r / 2), half = r % 2;

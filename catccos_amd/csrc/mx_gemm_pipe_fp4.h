@@ -233,9 +233,9 @@ __global__ __launch_bounds__(256) void mx_gemm_pipe_fp4_kernel(const GemmParams 
 #define CMX_PIPE_WOFF(f) ((epi_pairs_gate_up(EPI) ? ((f) < FW / 2 ? (f) * 32 : TW / 2 + ((f) - FW / 2) * 32) : (f) * 32))
     auto read_piece = [&](auto slot_c, auto step_c, auto pos_c, v4i (&f)[NF]) {
         constexpr int slot = decltype(slot_c)::value, step = decltype(step_c)::value;
-        // the last step's fragments of a slot are read weights first in the persistent 2 x 2 kernels, so that the weight rows
+        // the last step's fragments of a slot are read weights first in the grouped kernels, so that the weight rows
         // are free (and their loads go out) while the activation fragments are still being read
-        constexpr int idx = (kPf > 0 && step == 3) ? decltype(pos_c)::value : pipe_read_order<FW, FM>(decltype(pos_c)::value);
+        constexpr int idx = ((kPf > 0 || kSkip) && step == 3) ? decltype(pos_c)::value : pipe_read_order<FW, FM>(decltype(pos_c)::value);
         (void)wb, (void)ab;
         if constexpr (idx < FW) f[idx] = lds_read_b128<CMX_PIPE_WOFF(idx) * kSlabBytes>(wb[slot][step]);
         else f[idx] = lds_read_b128<(idx - FW) * 32 * kSlabBytes>(ab[slot][step]);
@@ -322,7 +322,7 @@ __global__ __launch_bounds__(256) void mx_gemm_pipe_fp4_kernel(const GemmParams 
 
     constexpr int kB1 = 9;                      // MFMA of step 2 after which the reads of step 3 have landed
     constexpr int kEarly = kM - kB1 - 1;        // tile loads of slab s+2 issued in step 2 (6)
-    constexpr bool kWFirst = kPf > 0;           // persistent 2 x 2 kernels: the eight weight loads go out early instead (see read_piece)
+    constexpr bool kWFirst = kPf > 0 || kSkip;  // grouped kernels: the eight weight loads go out early instead (see read_piece)
     constexpr int kEarlyN = kWFirst ? kWTileLoads : kEarly;
     constexpr uint32_t kNoSlab = 0xFFFFFFFFu;
     // q = slab of the load stream within its tile (kNoSlab: nothing new to request, slab q2 is requested again)

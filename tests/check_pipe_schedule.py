@@ -53,10 +53,10 @@ KERNELS = [
     ("mx_gemm_pipe_kernel<0, 1, 128, 4, 1, 3>", {14}),
     ("mx_gemm_pipe_fp4_kernel<2, 2, 2>", {10}),
     ("mx_gemm_pipe_fp4_kernel<4, 2, 2>", {10}),
-    ("mx_gemm_pipe_fp4_kernel<2, 4, 1>", {6}),
-    ("mx_gemm_pipe_fp4_kernel<4, 4, 1>", {6}),
+    ("mx_gemm_pipe_fp4_kernel<2, 4, 1>", {8}),
+    ("mx_gemm_pipe_fp4_kernel<4, 4, 1>", {8}),
     ("mx_gemm_pipe_fp4_kernel<0, 2, 2>", {6}),
-    ("mx_gemm_pipe_fp4_kernel<0, 4, 1>", {6}),
+    ("mx_gemm_pipe_fp4_kernel<0, 4, 1>", {8}),
 ]
 
 
