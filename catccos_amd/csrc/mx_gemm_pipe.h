@@ -17,7 +17,10 @@
 //           flight) and a second barrier that makes slab s+1 visible to all.
 //   step 1: 16 MFMAs on fragment set 1.  Behind them the other 9+2 loads of slab s+2, the 16 reads of
 //           fragment set 0 from slab s+1, its 8 scale dwords and their per-half-wave byte shift.
-// A load is thus in flight for 23 to 38 MFMA times before anyone waits for it.
+// A load is thus in flight for 23 to 38 MFMA times before anyone waits for it.  (The grouped two-slot kernels read the
+// second half's weight fragments first, free the weight rows of the slot with a barrier after MFMA 4 (2 x 2) or 2 (4 x 1)
+// and send all eight weight loads of slab s+2 behind the following MFMAs; the persistent 2 x 2 kernels also issue two L2
+// prefetch loads per slab in step 1: see kWFirst and CMX_PIPE_PREFETCH below.)
 // Every LDS address is a per-lane base register plus an immediate, every global address a per-lane
 // offset register plus a scalar slab offset: the loop contains no address arithmetic on the VALU.
 #pragma once
