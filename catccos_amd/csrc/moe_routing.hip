@@ -482,6 +482,12 @@ __global__ __launch_bounds__(256) void int8_quant_scatter_kernel(const uint16_t*
 }  // namespace
 }  // namespace cmx
 
+int cmx::preload_routing_kernels() {
+    hipFuncAttributes attr;
+    CMX_HIP(hipFuncGetAttributes(&attr, reinterpret_cast<const void*>(cmx::route_hist_kernel)));
+    return CMX_OK;
+}
+
 extern "C" size_t cmx_moe_routing_workspace_bytes(uint32_t routes, uint32_t experts) {
     const size_t chunks = (routes + cmx::kChunk - 1) / cmx::kChunk;
     return cmx::round_up_sz((chunks ? chunks : 1) * (size_t)experts * sizeof(uint32_t), 256);
@@ -536,12 +542,16 @@ extern "C" int cmx_quant_scatter(const void* x, uint32_t ld_x, const int32_t* sr
     const uint16_t* xp = static_cast<const uint16_t*>(x);
     hipStream_t s = static_cast<hipStream_t>(stream);
     // Scale rows that can be written in 16-byte pieces take the row-wise kernel: the row, its padding column and zeros
-    // up to a multiple of 16 bytes -- or up to the whole pitch when that is the next multiple of 128 (then every
-    // 128-byte line of the scale array is written whole).  Bytes of a row behind its scale_cols(k) columns belong
-    // to the pitch, not to the data, and callers must not keep anything there.
+    // up to a multiple of 16 bytes (never beyond: in the packed wire row, whose scale bytes sit behind the codes of the
+    // same row, round_up(scale_cols, 16) <= round_up(scale_cols, 32) = the bytes the row has left behind its codes).
+    // Only a scale array that is an allocation of its own -- one that does not overlap the code rows -- gets whole
+    // pitches written when the pitch is the next multiple of 128, so that every 128-byte line of it is written whole.
     const uint32_t run16 = round_up(scale_cols(k), 16);
     if (ld_outs % 16 == 0 && aligned16(out_scales) && run16 <= ld_outs && nb <= 1024) {
-        const uint32_t run = ld_outs == round_up(scale_cols(k), 128) ? ld_outs : run16;
+        const uint64_t dst_rows = (uint64_t)tokens * top_k;
+        const uintptr_t c0 = reinterpret_cast<uintptr_t>(out_codes), s0 = reinterpret_cast<uintptr_t>(out_scales);
+        const bool disjoint = s0 >= c0 + dst_rows * ld_out || s0 + dst_rows * ld_outs <= c0;
+        const uint32_t run = (disjoint && ld_outs == round_up(scale_cols(k), 128)) ? ld_outs : run16;
         hipLaunchKernelGGL(quant_scatter_row_kernel, dim3(tokens), dim3(256), 0, s, xp, ld_x, src2sorted, out_codes, ld_out,
                            out_scales, ld_outs, top_k, nb, run);
         CMX_LAUNCH_CHECK();

@@ -40,6 +40,13 @@ void set_error(const std::string& msg);
         }                                                                                        \
     } while (0)
 
+// Each translation unit with kernels is a code object of its own, loaded on a device when one of its kernels is first
+// looked up there.  cmx_init calls these so that no later launch -- possibly one inside a stream capture -- is the
+// first to do so.  Each asks the runtime for the attributes of one kernel of its unit on the current device.
+int preload_routing_kernels();
+int preload_layout_kernels();
+int preload_quant_kernels();
+
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 inline uint32_t ceil_div(uint32_t a, uint32_t b) { return (a + b - 1) / b; }
 inline uint32_t round_up(uint32_t a, uint32_t b) { return ceil_div(a, b) * b; }

@@ -1456,13 +1456,20 @@ extern "C" int cmx_mx_gmm_swiglu_quant_noalloc(const uint8_t* a, uint32_t lda, c
                             group_sizes, groups, m_total, n, k, meta, stream);
 }
 
-// One-time set-up on the current device: raises the dynamic-LDS limit of every matmul kernel, reads the CU count and
-// resolves the static schedule array, so that no later call has to (none of this is allowed, or wise, inside a
-// stream capture).  Optional: every entry point still does what it needs on first use.
+// One-time set-up on the current device: raises the dynamic-LDS limit of every matmul kernel, has the runtime load the
+// code object of every translation unit, reads the CU count and resolves the static schedule array, so that no later
+// call has to (none of this is allowed, or wise, inside a stream capture).  Optional: every entry point still does
+// what it needs on first use.
 extern "C" int cmx_init(void) {
     using namespace cmx;
     for (const LdsKernel& k : lds_registry())
         if (int rc = allow_dynamic_lds(k.fn, k.bytes, *k.flag); rc != CMX_OK) return rc;
+    // the matmul kernels without an LDS limit to raise (and with them this unit's code object), then the other units
+    hipFuncAttributes attr;
+    CMX_HIP(hipFuncGetAttributes(&attr, reinterpret_cast<const void*>(gmm_prepare_kernel)));
+    if (int rc = preload_routing_kernels(); rc != CMX_OK) return rc;
+    if (int rc = preload_layout_kernels(); rc != CMX_OK) return rc;
+    if (int rc = preload_quant_kernels(); rc != CMX_OK) return rc;
     int cus = 0;
     if (int rc = cu_count(&cus); rc != CMX_OK) return rc;
     void* meta = nullptr;

@@ -347,6 +347,12 @@ int normalise(const uint8_t* src, const uint8_t* src_scale, uint8_t* dst, uint8_
 }  // namespace
 }  // namespace cmx
 
+int cmx::preload_layout_kernels() {
+    hipFuncAttributes attr;
+    CMX_HIP(hipFuncGetAttributes(&attr, reinterpret_cast<const void*>(cmx::mx_to_k_major16_kernel)));
+    return CMX_OK;
+}
+
 extern "C" int cmx_mx_to_k_major(const uint8_t* src, uint32_t ld_src, const uint8_t* src_scale, uint8_t* dst,
                                  uint32_t ld_dst, uint8_t* dst_scale, uint32_t ld_dst_scale, uint32_t k, uint32_t n,
                                  uint32_t batch, cmx_stream_t stream) {

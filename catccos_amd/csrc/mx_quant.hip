@@ -255,6 +255,12 @@ int launch_quant(bool lut, dim3 grid, hipStream_t s, const uint16_t* x, uint32_t
 
 }  // namespace cmx
 
+int cmx::preload_quant_kernels() {
+    hipFuncAttributes attr;
+    CMX_HIP(hipFuncGetAttributes(&attr, reinterpret_cast<const void*>(cmx::mx_dequant_kernel)));
+    return CMX_OK;
+}
+
 extern "C" int cmx_mx_quant(const void* x, uint32_t ld_x, uint8_t* codes, uint32_t ld_codes, uint8_t* scales,
                             uint32_t ld_scales, uint32_t rows, uint32_t cols, int fmt, int round_mode,
                             cmx_stream_t stream) {

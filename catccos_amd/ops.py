@@ -232,17 +232,19 @@ def moe_init_routing(expert_idx: torch.Tensor, experts: int):
     return s2s, inv, counts
 
 
-def quant_scatter(x: torch.Tensor, src2sorted: torch.Tensor, top_k: int, packed: bool = False):
+def quant_scatter(x: torch.Tensor, src2sorted: torch.Tensor, top_k: int, packed: bool = False, out=None):
     """x bf16 [T, k] -> rows quantised once and written to their top_k destinations.
     packed=False: (codes [T*topK, k], scales [T*topK, RoundUp2(k/32)]);
-    packed=True: one buffer [T*topK, packed_row_bytes(k)] = codes | scales | pad."""
+    packed=True: one buffer [T*topK, packed_row_bytes(k)] = codes | scales | pad (``out``: a caller's zeroed buffer
+    of that shape)."""
     _need_cuda(x, src2sorted)
     t, k = x.shape
     rows = t * top_k
     lib = _lib.load()
     if packed:
         rb = lib.cmx_packed_row_bytes(k)
-        buf = torch.zeros((rows, rb), dtype=torch.uint8, device=x.device)
+        buf = torch.zeros((rows, rb), dtype=torch.uint8, device=x.device) if out is None else out
+        assert buf.shape == (rows, rb) and buf.dtype == torch.uint8 and buf.is_contiguous()
         _lib.check(lib.cmx_quant_scatter(_p(x), x.stride(0), _p(src2sorted), _p(buf), rb, buf.data_ptr() + k, rb, t, k,
                                          top_k, _stream()))
         return buf

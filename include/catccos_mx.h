@@ -267,11 +267,17 @@ int cmx_moe_init_routing(const int32_t* expert_idx, uint32_t tokens, uint32_t to
  *
  *   x           bf16 [tokens, k]
  *   src2sorted  int32 [tokens*top_k]; negative destinations are skipped
- *   out_codes   row r at out_codes + r*ld_out (16-byte aligned rows);  out_scales row r at out_scales + r*ld_outs.
- *               Bytes of a scale row behind its RoundUp2(k/32) columns, up to the pitch, may be overwritten with zeros
- *               (scale rows are written in 16-byte pieces, whole 128-byte lines when the pitch is the next multiple of 128).
- * The reference's packed wire row [codes k | scales RoundUp2(k/32) | pad to 32 B] is the case
- * out_scales = out_codes + k, ld_out = ld_outs = cmx_packed_row_bytes(k).
+ *   out_codes   row r at out_codes + r*ld_out; rows 16-byte aligned (ld_out a multiple of 16).
+ *   out_scales  row r at out_scales + r*ld_outs.  When the scale rows are 16-byte aligned too they are written in
+ *               16-byte pieces: the bytes of a row between its RoundUp2(k/32) columns and the next multiple of 16
+ *               are overwritten with zeros, never more -- unless the scale array is an allocation of its own (it
+ *               does not overlap [out_codes, out_codes + tokens*top_k*ld_out)) and ld_outs is the next multiple of
+ *               128: then the whole pitch is written (data, padding column, zeros), so that no 128-byte line of
+ *               the array is written in part.  Callers keep nothing in those bytes.
+ * The reference's packed wire row [codes k | scales RoundUp2(k/32) | zero pad to 32 B] is the case
+ * out_scales = out_codes + k, ld_out = ld_outs = cmx_packed_row_bytes(k): the zero fill then ends at or before the
+ * end of the row's own pad bytes (k is a multiple of 32, so the row has round_up(RoundUp2(k/32), 32) bytes behind
+ * its codes), whatever k is.
  * ---------------------------------------------------------------------------------------- */
 uint32_t cmx_packed_row_bytes(uint32_t k);
 int cmx_quant_scatter(const void* x, uint32_t ld_x, const int32_t* src2sorted, uint8_t* out_codes, uint32_t ld_out,

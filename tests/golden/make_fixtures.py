@@ -15,6 +15,13 @@ What is imported, and why each needs the real thing rather than a restatement:
   the FFN chain (which half of GMM1 gets the SiLU, where the bf16 roundings sit, which quantizer rounding each
   operand gets, how the combine accumulates).
 
+* ``examples/ascend950_mxfp8_matmul_reduce_scatter/scripts/gen_data_mxfp8_mmrs.py`` -- ``gen_data`` on a tiny shape, B
+  stored both ways: the operand and scale FILE layouts of the dense MXFP8 example ([K, N] codes with [K/64, N, 2]
+  scales, and the transposed pair), its per-element E5M2 table quantizer and its ``golden`` / ``golden_low`` pair.
+* ``examples/utils/gen_data_fp4_mx_alltoallv_gmm.py`` -- ``generate_data`` on a tiny shape: the legacy
+  ``MXFP4MatrixQuantizer`` (E2M1 table rounding, bit-level nibble packing), the file layouts of the FP4 grouped-matmul
+  example and its fp32 golden.
+
 ``gen_data_dispatch_gmm_dequant_swiglu.py`` is not imported (it needs an NPU-only package and deletes
 ``./output`` at import time).
 """
@@ -151,6 +158,49 @@ def main() -> int:
         )
     np.savez_compressed(os.path.join(HERE, "ffn_tiny.npz"), **ffn)
     print("wrote ffn_tiny.npz:", ", ".join(f"{a}{tuple(v.shape)}" for a, v in ffn.items()))
+
+    # ---- dense MXFP8 matmul example: file layouts and the double golden ------------------------------------------
+    sys.path.insert(0, os.path.join(ref, "examples", "ascend950_mxfp8_matmul_reduce_scatter", "scripts"))
+    import gen_data_mxfp8_mmrs as D                                 # noqa: E402  (reference module)
+    m, k, n = 8, 128, 16
+    mm = dict(shape=np.array([m, k, n], dtype=np.int64))
+    torch.manual_seed(11)                                           # gen_data draws A [m, k], then B [k, n]
+    mm["a_src"] = torch.randn((m, k), dtype=torch.float32).numpy().copy()
+    mm["b_src"] = torch.randn((k, n), dtype=torch.float32).numpy().copy()
+    for trans_b in (1, 0):                                          # 1 is what the example's run.sh passes
+        torch.manual_seed(11)                                       # the same random matrices for both orientations
+        with tempfile.TemporaryDirectory() as tmp:
+            c_fp32, c_bf16 = D.gen_data(0, m, k, n, 0, trans_b, tmp)
+            for what in ("a", "b", "a_scale", "b_scale"):
+                mm[f"tb{trans_b}_{what}"] = np.fromfile(os.path.join(tmp, f"rank_0_{what}.bin"), dtype=np.uint8)
+        mm[f"tb{trans_b}_golden"] = c_fp32.numpy().copy()
+        mm[f"tb{trans_b}_golden_low"] = c_bf16.view(torch.uint16).numpy().copy()
+    np.savez_compressed(os.path.join(HERE, "mmrs_tiny.npz"), **mm)
+    print("wrote mmrs_tiny.npz:", ", ".join(f"{a}{tuple(v.shape)}" for a, v in mm.items()))
+
+    # ---- FP4 grouped matmul example ---------------------------------------------------------------------------------
+    import argparse
+    import gen_data_fp4_mx_alltoallv_gmm as F                       # noqa: E402  (reference module)
+    from utils import DataType                                      # noqa: E402  (reference module)
+    m, k, n, experts = 24, 128, 32, 3
+    torch.manual_seed(12)                                           # generate_data draws A [1, m, k], then B [1, E, k, n]
+    a_src = F.random_uniform(-2.0, 2.0, size=(1, m, k)).numpy().copy()[0]
+    b_src = F.random_uniform(-2.0, 2.0, size=(1, experts, k, n)).numpy().copy()[0]
+    torch.manual_seed(12)
+    with tempfile.TemporaryDirectory() as tmp:
+        F.generate_data(argparse.Namespace(out_type=DataType.FLOAT16, rank_size=1, m=m, n=n, k=k, trans_a=0, trans_b=0,
+                                           expert=experts, ep=1, data_dir=tmp))
+        rd = lambda name, dtype: np.fromfile(os.path.join(tmp, name), dtype=dtype)
+        f4 = dict(
+            shape=np.array([m, k, n, experts], dtype=np.int64), a_src=a_src, b_src=b_src,
+            input_a=rd("input_a_0.bin", np.uint8), input_a_scale=rd("input_a_scale_0.bin", np.uint8),
+            input_b=rd("input_b_0.bin", np.uint8), input_b_scale=rd("input_b_scale_0.bin", np.uint8),
+            local_tokens_per_expert=rd("local_tokens_per_expert_0.bin", np.int32),
+            global_tokens_per_local_expert=rd("global_tokens_per_local_expert_0.bin", np.int32),
+            golden=rd("golden_0.bin", np.float32).reshape(m, n),
+        )
+    np.savez_compressed(os.path.join(HERE, "fp4_gmm_tiny.npz"), **f4)
+    print("wrote fp4_gmm_tiny.npz:", ", ".join(f"{a}{tuple(v.shape)}" for a, v in f4.items()))
     return 0
 
 

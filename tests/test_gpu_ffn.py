@@ -151,3 +151,14 @@ def test_ffn_chain_replays_from_a_hip_graph():
         graph.replay()
         torch.cuda.synchronize()
         assert torch.equal(out.view(torch.int16), expect.view(torch.int16)), rep
+
+
+def test_capture_right_after_init():
+    """A process whose first launches of the library's kernels happen inside a stream capture, after cmx_init() alone
+    (tests/capture_after_init_child.py): the FFN chain and the allocation-free grouped matmul replay bit for bit."""
+    import os
+    import subprocess
+    import sys
+    child = os.path.join(os.path.dirname(os.path.abspath(__file__)), "capture_after_init_child.py")
+    r = subprocess.run([sys.executable, child], capture_output=True, text=True, timeout=300)
+    assert r.returncode == 0 and "CAPTURE-OK" in r.stdout, (r.returncode, r.stdout[-2000:], r.stderr[-2000:])

@@ -54,6 +54,29 @@ def test_quant_scatter_bit_exact(packed):
         assert np.array_equal(host(codes), want[:, :k]) and np.array_equal(host(scales), want[:, k:k + k // 32])
 
 
+@pytest.mark.parametrize("k", [64, 96, 480, 512, 4064])
+def test_quant_scatter_packed_rows_touch_nothing_else(k):
+    """The packed wire layout (scale bytes behind the codes of the same row): every byte of the buffer is the oracle's,
+    pad bytes included, and the bytes in front of the first and behind the last row keep their fill.  k = 96 is the case
+    whose packed row (128 bytes) equals the scale row rounded up to a whole 128-byte line."""
+    from catccos_amd import ops
+    tokens, top_k, experts, guard = 40, 3, 6, 4
+    rng = np.random.default_rng(k)
+    xb = W.activations_with_outliers(tokens, k, seed=k + 1)
+    idx = np.stack([rng.permutation(experts)[:top_k] for _ in range(tokens)]).astype(np.int32)
+    _, inv, _ = O.moe_init_routing(idx, experts)
+    want = O.quant_scatter_packed(xb, inv, top_k)
+    rows, rb = want.shape
+    assert rb == O.packed_row_bytes(k)
+    whole = torch.full((rows + 2 * guard, rb), 0xA5, dtype=torch.uint8, device="cuda")
+    mid = whole[guard:guard + rows]
+    mid.zero_()
+    ops.quant_scatter(bf16_dev(xb), dev(inv), top_k, packed=True, out=mid)
+    got = host(whole)
+    assert np.array_equal(got[guard:guard + rows], want)
+    assert np.all(got[:guard] == 0xA5) and np.all(got[guard + rows:] == 0xA5)
+
+
 @pytest.mark.parametrize("k", [512, 7168, 96])
 def test_quant_scatter_non_finite_tokens_equal_the_quantizer(k):
     """Tokens with Inf / NaN elements through both scatter kernels (k = 96: scale rows that are not 16-byte aligned take the
