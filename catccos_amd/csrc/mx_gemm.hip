@@ -67,6 +67,7 @@ struct GemmParams {
     int out_type;
     int scale_vec;   // scale rows are 4-byte aligned: one dword load per row and slab
     int scale_vec16; // scale rows are 16-byte aligned: one 16-byte load per row fetches the scales of four slabs
+    int w_pretiled;  // w holds the weights in the tiled order of cmx_mx_pretile_weights (the weights-to-registers kernel)
 };
 
 __device__ __forceinline__ uint32_t swz(uint32_t row, uint32_t chunk) {
@@ -883,6 +884,7 @@ __global__ __launch_bounds__(64 * WW * WM) void mx_gemm_dl_kernel(const GemmPara
 }
 
 #include "mx_gemm_pipe.h"
+#include "mx_gemm_wreg.h"
 #include "mx_gemm_pipe_fp4.h"
 
 // Row offsets and m-tile prefix of the groups (one workgroup of 256 threads): each thread owns a contiguous run of
@@ -1062,6 +1064,26 @@ int launch_gemm_pipe(const GemmParams& p, uint32_t max_m_tiles, hipStream_t s) {
     return CMX_OK;
 }
 
+template <int FMT, int EPI>
+int launch_gemm_wreg(const GemmParams& p, uint32_t max_m_tiles, hipStream_t s) {
+    // activation ring (four 32 KiB slots), ring of two scale blocks (16 bytes per row of both operands), next-tile mailbox
+    constexpr size_t smem = 4 * 256 * kSlabBytes + 2 * 512 * 16 + 512;
+    constexpr auto kfn = mx_gemm_wreg_kernel<FMT, EPI, false>;
+    constexpr auto kfn_pre = mx_gemm_wreg_kernel<FMT, EPI, true>;
+    if (int rc = allow_dynamic_lds<kfn, smem>(); rc != CMX_OK) return rc;
+    if (int rc = allow_dynamic_lds<kfn_pre, smem>(); rc != CMX_OK) return rc;
+    const uint64_t tiles = (uint64_t)max_m_tiles * p.w_tiles;
+    CMX_REQUIRE(tiles > 0 && tiles < (1ull << 31), "tile count out of range");
+    int cus = 0;
+    if (int rc = cu_count(&cus); rc != CMX_OK) return rc;
+    uint32_t grid = (uint32_t)(cus / kXcds * kXcds);
+    if (grid < (uint32_t)kXcds) grid = kXcds;
+    if (p.w_pretiled) hipLaunchKernelGGL(kfn_pre, dim3(grid), dim3(256), smem, s, p);
+    else hipLaunchKernelGGL(kfn, dim3(grid), dim3(256), smem, s, p);
+    CMX_LAUNCH_CHECK();
+    return CMX_OK;
+}
+
 template <int EPI, int WW, int WM>
 int launch_gemm_pipe_fp4(const GemmParams& p, uint32_t max_m_tiles, hipStream_t s) {
     constexpr size_t smem = 2 * 512 * kSlabBytes + 2 * 512 * 16 + 512;    // tile ring, ring of two scale blocks, next-tile mailbox, sink of the L2 prefetch loads
@@ -1086,6 +1108,7 @@ int launch_gemm_pipe_fp4(const GemmParams& p, uint32_t max_m_tiles, hipStream_t 
 // kernels and pin the tile shape, so that tests reach every compiled instantiation; the product has neither switch.
 #ifdef CMX_TEST_HOOKS
 bool g_disable_dl = false;
+int g_w_pretiled = 0;
 #else
 constexpr bool g_disable_dl = false;
 #endif
@@ -1137,13 +1160,19 @@ int launch_tile(const GemmParams& p, int waves, uint32_t max_m_tiles, hipStream_
     const bool stream_ok = !g_disable_dl && p.scale_vec && p.kbytes % kSlabBytes == 0;
     if constexpr (TW == 256 && TM == 256 && FMT != CMX_FMT_E2M1) {
         // whole four-slab scale blocks, fetched 16 bytes per row: K a multiple of 512 bytes, 16-byte aligned scale rows
-        if ((waves == 4 || waves == 5) && stream_ok && p.scale_vec16 && p.kbytes % (4 * kSlabBytes) == 0) {
+        if ((waves == 4 || waves == 5 || waves == 6) && stream_ok && p.scale_vec16 && p.kbytes % (4 * kSlabBytes) == 0) {
             // plain 16-bit output with 8-element-aligned rows takes the lean store epilogue and with it the persistent kernel
             constexpr int kLeanBf16 = EPI == kEpiStore ? kEpiStoreBf16 : EPI, kLeanFp16 = EPI == kEpiStore ? kEpiStoreFp16 : EPI;
             const bool lean = EPI == kEpiStore && p.out_type != CMX_OUT_FP32 && p.n % 8 == 0 && p.ldc % 8 == 0 &&
                               (reinterpret_cast<uintptr_t>(p.c) & 15u) == 0;
             // (the 4 x 1 layout with the lean store epilogue does not fit the register file without spilling
             // inside the loop, so the persistent store kernel is always 2 x 2)
+            if constexpr (EPI != kEpiStore) {
+                if (waves == 6) return launch_gemm_wreg<FMT, EPI>(p, max_m_tiles, s);
+            } else {
+                if (waves == 6 && lean && p.out_type == CMX_OUT_BF16) return launch_gemm_wreg<FMT, kEpiStoreBf16>(p, max_m_tiles, s);
+                if (waves == 6 && lean) return launch_gemm_wreg<FMT, kEpiStoreFp16>(p, max_m_tiles, s);
+            }
             if (lean && p.out_type == CMX_OUT_BF16) return launch_gemm_pipe<FMT, kLeanBf16, 256, 2, 2, 2>(p, max_m_tiles, s);
             if (lean) return launch_gemm_pipe<FMT, kLeanFp16, 256, 2, 2, 2>(p, max_m_tiles, s);
             if (waves == 4) return launch_gemm_pipe<FMT, EPI, 256, 2, 2, 2>(p, max_m_tiles, s);
@@ -1219,6 +1248,11 @@ extern "C" int cmx_debug_disable_streaming(int off) {
     return CMX_OK;
 }
 
+extern "C" int cmx_debug_w_pretiled(int on) {
+    cmx::g_w_pretiled = on;
+    return CMX_OK;
+}
+
 // pin the tile shape and wavefront count of every later matmul call (tw = 0 restores the heuristic)
 extern "C" int cmx_debug_force_tile(int tw, int tm, int waves) {
     cmx::g_force_tile = (tw > 0 && tm > 0) ? cmx::TileChoice{tw, tm, waves > 0 ? waves : 4} : cmx::TileChoice{0, 0, 0};
@@ -1277,12 +1311,18 @@ int gmm_common(GemmParams& p, const int32_t* group_sizes, uint32_t groups, uint3
     hipLaunchKernelGGL(gmm_prepare_kernel, dim3(1), dim3(256), 0, s, group_sizes, groups, (uint32_t)t.tm, m_total, row_off,
                        tile_pref, tile_ctr);
     CMX_LAUNCH_CHECK();
+#ifdef CMX_TEST_HOOKS
+    p.w_pretiled = g_w_pretiled & 1;
+#endif
     p.row_off = row_off;
     p.tile_pref = tile_pref;
     // The persistent kernels draw their next tile from a per-XCD counter when tiles differ in cost (4 x 1 wavefronts skip
     // the MFMAs of absent rows).  With 2 x 2 wavefronts every tile costs the same, so those kernels walk their XCD's run in
     // fixed strides instead: no atomic whose result has to be waited for with everything else in flight.
     p.tile_ctr = t.waves == 4 ? nullptr : tile_ctr;
+#ifdef CMX_TEST_HOOKS
+    if (g_w_pretiled & 2) p.tile_ctr = nullptr;
+#endif
     p.groups = groups;
     p.w_tiles = swiglu ? ceil_div(p.n / 2, t.tw / 2) : ceil_div(p.n, t.tw);
     const uint32_t max_m_tiles = m_total / t.tm + groups;
