@@ -394,8 +394,21 @@ def main() -> int:
             stages["quant_scatter"].update({"hbm_frac": b_qs4 / (acc_ms[1] * 1e-3) / 1e9 / HBM_PEAK_GBS})
             stages["unpermute_combine"].update({"hbm_frac": b_c4 / (acc_ms[4] * 1e-3) / 1e9 / HBM_PEAK_GBS})
             log("[moe ffn cfg4 stages] " + ", ".join(f"{n} {v['us']:.0f} us" for n, v in stages.items()))
-            del ac, asc, hc, hs, yy
-            extra["moe_ffn_cfg4"] = {"ms": tf * 1e3, "stages_in_chain": stages, "tflops": fl4 / tf / 1e12, "mfma_frac": fl4 / tf / 1e12 / MXFP8_PEAK_TFLOPS,
+            # the same chain on weights pre-tiled once at load time (cmx_mx_pretile_weights): both matmuls then run the
+            # weights-to-registers kernel; "ms" stays the figure of the reference's own entry point on row-major weights
+            t0 = time.perf_counter()
+            w14t, w24t = ops.pretile_weights(w14, True), ops.pretile_weights(w24, False)
+            torch.cuda.synchronize()
+            t_tile = time.perf_counter() - t0
+            tft = hip_time(lambda: ops.dispatch_ffn_combine(x4, idx4_d, p4_d, w14t, w14s, w24t, w24s, workspace=wsp, out=out4),
+                           steps=max(5, K_STEPS // 2), warm=2)
+            tg1 = hip_time(lambda: ops.mx_gmm_swiglu_quant(ac, asc, w14t, w14s, cnt4b, K4, workspace=gw1, outs=(hc, hs)), steps=5, warm=2)
+            tg2 = hip_time(lambda: ops.mx_gmm(hc, hs, w24t, w24s, cnt4b, N4 // 2, "E4M3", "bf16", c=yy, workspace=gw2), steps=5, warm=2)
+            pre = {"ms": tft * 1e3, "gmm1_swiglu_requant_us": tg1 * 1e6, "gmm2_us": tg2 * 1e6, "pretile_pass_ms_once": t_tile * 1e3,
+                   "tflops": fl4 / tft / 1e12, "hbm_frac": by4 / tft / 1e9 / HBM_PEAK_GBS}
+            log(f"[moe ffn cfg4, pre-tiled weights] {tft*1e3:.3f} ms (gmm1 {tg1*1e6:.0f} us, gmm2 {tg2*1e6:.0f} us back to back; tiling pass once {t_tile*1e3:.1f} ms)")
+            del ac, asc, hc, hs, yy, w14t, w24t
+            extra["moe_ffn_cfg4"] = {"ms": tf * 1e3, "pretiled_weights": pre, "stages_in_chain": stages, "tflops": fl4 / tf / 1e12, "mfma_frac": fl4 / tf / 1e12 / MXFP8_PEAK_TFLOPS,
                                      "algorithmic_GB": by4 / 1e9, "hbm_GBs": by4 / tf / 1e9, "hbm_frac": by4 / tf / 1e9 / HBM_PEAK_GBS,
                                      "tokens_per_s": T4 / tf}
             log(f"[moe ffn cfg4] {tf*1e3:.3f} ms -> {fl4/tf/1e12:.0f} TFLOP/s, {by4/tf/1e9:.0f} GB/s algorithmic")

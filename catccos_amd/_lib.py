@@ -69,6 +69,13 @@ SIGNATURES = {
     "catccos_ascend950_dispatch_ffn_combine": (i32, [u32, vp, u64, u8p, u8p, u8p, u8p, u8p, u8p, u8p, u8p, u8p, u8p,
                                                      u32, u32, u32, u32, u32, i32]),
     "cmx_ffn_workspace_layout_get": (i32, [u32, u32, u32, u32, u32, C.POINTER(FfnWorkspaceLayout)]),
+    "cmx_mx_pretiled_weight_bytes": (sz, [u32, u32, u32, i32]),
+    "cmx_mx_pretile_weights": (i32, [u8p, u8p, u32, u32, u32, i32, vp]),
+    "cmx_mx_gmm_pretiled": (i32, [u8p, u32, u8p, u32, u8p, u8p, vp, u32, i32p, u32, u32, u32, u32, i32, i32, vp, vp]),
+    "cmx_mx_gmm_swiglu_quant_pretiled": (i32, [u8p, u32, u8p, u32, u8p, u8p, u8p, u32, u8p, u32, vp, i32p, u32, u32,
+                                               u32, u32, vp, vp]),
+    "cmx_dispatch_ffn_combine_pretiled": (i32, [vp, u8p, u8p, u8p, u8p, u8p, u8p, u8p, u8p, u8p, u32, u32, u32, u32,
+                                                u32]),
     "cmx_init": (i32, []),
     "cmx_mx_gmm_noalloc_max_groups": (u32, []),
     "cmx_mx_gmm_swiglu_quant_noalloc": (i32, [u8p, u32, u8p, u32, u8p, u8p, u8p, u32, u8p, u32, vp, i32p, u32, u32, u32,

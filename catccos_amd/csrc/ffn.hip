@@ -72,24 +72,18 @@ extern "C" size_t catccos_ascend950_dispatch_ffn_combine_workspace_bytes(uint32_
     return L.total;
 }
 
-extern "C" int catccos_ascend950_dispatch_ffn_combine(uint32_t blockDim, cmx_stream_t stream, uint64_t fftsAddr,
-                                                      const uint8_t* x, const uint8_t* expertIdx,
-                                                      const uint8_t* gateWeight, const uint8_t* w1,
-                                                      const uint8_t* w1Scale, const uint8_t* w2, const uint8_t* w2Scale,
-                                                      uint8_t* out, uint8_t* workspace, uint8_t* symmetric, uint32_t m,
-                                                      uint32_t k, uint32_t n, uint32_t localExperts, uint32_t topK,
-                                                      int rankSize) {
-    using namespace cmx;
-    (void)blockDim;
-    (void)fftsAddr;
-    (void)symmetric;
-    CMX_REQUIRE(rankSize == 1, "one device only: rankSize must be 1");
+namespace cmx {
+namespace {
+int ffn_chain(cmx_stream_t stream, const uint8_t* x, const uint8_t* expertIdx, const uint8_t* gateWeight, const uint8_t* w1,
+              const uint8_t* w1Scale, const uint8_t* w2, const uint8_t* w2Scale, uint8_t* out, uint8_t* workspace, uint32_t m,
+              uint32_t k, uint32_t n, uint32_t localExperts, uint32_t topK, bool pretiled) {
     CMX_REQUIRE(x && expertIdx && gateWeight && w1 && w1Scale && w2 && w2Scale && out && workspace, "null pointer");
     CMX_REQUIRE(m > 0 && localExperts > 0 && topK > 0 && topK <= localExperts, "bad routing shape");
     // limits of the stages further down the chain, checked before anything is launched
     CMX_REQUIRE(topK <= 64, "topK must not exceed 64 (weighted combine)");
     CMX_REQUIRE((uint64_t)m * topK < (1ull << 31), "m * topK must stay below 2^31 routes");
     CMX_REQUIRE(k % 256 == 0 && n % 512 == 0, "MXFP8 FFN requires K % 256 == 0 and N % 512 == 0");
+    CMX_REQUIRE(!pretiled || (k % 512 == 0 && n % 1024 == 0), "pre-tiled weights require K % 512 == 0 and N % 1024 == 0");
     CMX_REQUIRE((reinterpret_cast<uintptr_t>(workspace) & 255u) == 0, "workspace must be 256-byte aligned");
     cmx_ffn_workspace_layout L;
     layout(m, k, n, localExperts, topK, &L);
@@ -111,12 +105,44 @@ extern "C" int catccos_ascend950_dispatch_ffn_combine(uint32_t blockDim, cmx_str
     const uint32_t ld_as = (uint32_t)L.a_scales_pitch;
     rc = cmx_quant_scatter(x, k, src2sorted, a_codes, k, a_scales, ld_as, m, k, topK, stream);
     if (rc != CMX_OK) return rc;
-    rc = cmx_mx_gmm_swiglu_quant(a_codes, k, a_scales, ld_as, w1, w1Scale, act_codes, n / 2, act_scales,
-                                 scale_cols(n / 2), nullptr, counts, localExperts, rows, n, k, meta1, stream);
+    const uint32_t ld_acts = scale_cols(n / 2);
+    rc = pretiled ? cmx_mx_gmm_swiglu_quant_pretiled(a_codes, k, a_scales, ld_as, w1, w1Scale, act_codes, n / 2, act_scales,
+                                                     ld_acts, nullptr, counts, localExperts, rows, n, k, meta1, stream)
+                  : cmx_mx_gmm_swiglu_quant(a_codes, k, a_scales, ld_as, w1, w1Scale, act_codes, n / 2, act_scales, ld_acts,
+                                            nullptr, counts, localExperts, rows, n, k, meta1, stream);
     if (rc != CMX_OK) return rc;
-    rc = cmx_mx_gmm(act_codes, n / 2, act_scales, scale_cols(n / 2), w2, w2Scale, y, k, counts, localExperts, rows, k,
-                    n / 2, CMX_FMT_E4M3, CMX_OUT_BF16, meta2, stream);
+    rc = pretiled ? cmx_mx_gmm_pretiled(act_codes, n / 2, act_scales, ld_acts, w2, w2Scale, y, k, counts, localExperts, rows, k,
+                                        n / 2, CMX_FMT_E4M3, CMX_OUT_BF16, meta2, stream)
+                  : cmx_mx_gmm(act_codes, n / 2, act_scales, ld_acts, w2, w2Scale, y, k, counts, localExperts, rows, k, n / 2,
+                               CMX_FMT_E4M3, CMX_OUT_BF16, meta2, stream);
     if (rc != CMX_OK) return rc;
     return cmx_moe_token_unpermute(y, k, rows, src2sorted, reinterpret_cast<const float*>(gateWeight), out, k, m, k,
                                    topK, stream);
+}
+}  // namespace
+}  // namespace cmx
+
+extern "C" int catccos_ascend950_dispatch_ffn_combine(uint32_t blockDim, cmx_stream_t stream, uint64_t fftsAddr,
+                                                      const uint8_t* x, const uint8_t* expertIdx,
+                                                      const uint8_t* gateWeight, const uint8_t* w1,
+                                                      const uint8_t* w1Scale, const uint8_t* w2, const uint8_t* w2Scale,
+                                                      uint8_t* out, uint8_t* workspace, uint8_t* symmetric, uint32_t m,
+                                                      uint32_t k, uint32_t n, uint32_t localExperts, uint32_t topK,
+                                                      int rankSize) {
+    using namespace cmx;
+    (void)blockDim;
+    (void)fftsAddr;
+    (void)symmetric;
+    CMX_REQUIRE(rankSize == 1, "one device only: rankSize must be 1");
+    return ffn_chain(stream, x, expertIdx, gateWeight, w1, w1Scale, w2, w2Scale, out, workspace, m, k, n, localExperts, topK,
+                     false);
+}
+
+extern "C" int cmx_dispatch_ffn_combine_pretiled(cmx_stream_t stream, const uint8_t* x, const uint8_t* expertIdx,
+                                                 const uint8_t* gateWeight, const uint8_t* w1_tiled, const uint8_t* w1Scale,
+                                                 const uint8_t* w2_tiled, const uint8_t* w2Scale, uint8_t* out,
+                                                 uint8_t* workspace, uint32_t m, uint32_t k, uint32_t n,
+                                                 uint32_t localExperts, uint32_t topK) {
+    return cmx::ffn_chain(stream, x, expertIdx, gateWeight, w1_tiled, w1Scale, w2_tiled, w2Scale, out, workspace, m, k, n,
+                          localExperts, topK, true);
 }

@@ -1066,20 +1066,16 @@ int launch_gemm_pipe(const GemmParams& p, uint32_t max_m_tiles, hipStream_t s) {
 
 template <int FMT, int EPI>
 int launch_gemm_wreg(const GemmParams& p, uint32_t max_m_tiles, hipStream_t s) {
-    // activation ring (four 32 KiB slots), ring of two scale blocks (16 bytes per row of both operands), next-tile mailbox
-    constexpr size_t smem = 4 * 256 * kSlabBytes + 2 * 512 * 16 + 512;
-    constexpr auto kfn = mx_gemm_wreg_kernel<FMT, EPI, false>;
-    constexpr auto kfn_pre = mx_gemm_wreg_kernel<FMT, EPI, true>;
-    if (int rc = allow_dynamic_lds<kfn, smem>(); rc != CMX_OK) return rc;
-    if (int rc = allow_dynamic_lds<kfn_pre, smem>(); rc != CMX_OK) return rc;
+    constexpr auto kfn = mx_gemm_wreg_kernel<FMT, EPI>;
+    if (int rc = allow_dynamic_lds<kfn, kWregLdsBytes>(); rc != CMX_OK) return rc;
     const uint64_t tiles = (uint64_t)max_m_tiles * p.w_tiles;
     CMX_REQUIRE(tiles > 0 && tiles < (1ull << 31), "tile count out of range");
+    // persistent: one workgroup per CU, a multiple of the XCD count
     int cus = 0;
     if (int rc = cu_count(&cus); rc != CMX_OK) return rc;
     uint32_t grid = (uint32_t)(cus / kXcds * kXcds);
     if (grid < (uint32_t)kXcds) grid = kXcds;
-    if (p.w_pretiled) hipLaunchKernelGGL(kfn_pre, dim3(grid), dim3(256), smem, s, p);
-    else hipLaunchKernelGGL(kfn, dim3(grid), dim3(256), smem, s, p);
+    hipLaunchKernelGGL(kfn, dim3(grid), dim3(256), kWregLdsBytes, s, p);
     CMX_LAUNCH_CHECK();
     return CMX_OK;
 }
@@ -1108,7 +1104,6 @@ int launch_gemm_pipe_fp4(const GemmParams& p, uint32_t max_m_tiles, hipStream_t 
 // kernels and pin the tile shape, so that tests reach every compiled instantiation; the product has neither switch.
 #ifdef CMX_TEST_HOOKS
 bool g_disable_dl = false;
-int g_w_pretiled = 0;
 #else
 constexpr bool g_disable_dl = false;
 #endif
@@ -1160,19 +1155,13 @@ int launch_tile(const GemmParams& p, int waves, uint32_t max_m_tiles, hipStream_
     const bool stream_ok = !g_disable_dl && p.scale_vec && p.kbytes % kSlabBytes == 0;
     if constexpr (TW == 256 && TM == 256 && FMT != CMX_FMT_E2M1) {
         // whole four-slab scale blocks, fetched 16 bytes per row: K a multiple of 512 bytes, 16-byte aligned scale rows
-        if ((waves == 4 || waves == 5 || waves == 6) && stream_ok && p.scale_vec16 && p.kbytes % (4 * kSlabBytes) == 0) {
+        if ((waves == 4 || waves == 5) && stream_ok && p.scale_vec16 && p.kbytes % (4 * kSlabBytes) == 0) {
             // plain 16-bit output with 8-element-aligned rows takes the lean store epilogue and with it the persistent kernel
             constexpr int kLeanBf16 = EPI == kEpiStore ? kEpiStoreBf16 : EPI, kLeanFp16 = EPI == kEpiStore ? kEpiStoreFp16 : EPI;
             const bool lean = EPI == kEpiStore && p.out_type != CMX_OUT_FP32 && p.n % 8 == 0 && p.ldc % 8 == 0 &&
                               (reinterpret_cast<uintptr_t>(p.c) & 15u) == 0;
             // (the 4 x 1 layout with the lean store epilogue does not fit the register file without spilling
             // inside the loop, so the persistent store kernel is always 2 x 2)
-            if constexpr (EPI != kEpiStore) {
-                if (waves == 6) return launch_gemm_wreg<FMT, EPI>(p, max_m_tiles, s);
-            } else {
-                if (waves == 6 && lean && p.out_type == CMX_OUT_BF16) return launch_gemm_wreg<FMT, kEpiStoreBf16>(p, max_m_tiles, s);
-                if (waves == 6 && lean) return launch_gemm_wreg<FMT, kEpiStoreFp16>(p, max_m_tiles, s);
-            }
             if (lean && p.out_type == CMX_OUT_BF16) return launch_gemm_pipe<FMT, kLeanBf16, 256, 2, 2, 2>(p, max_m_tiles, s);
             if (lean) return launch_gemm_pipe<FMT, kLeanFp16, 256, 2, 2, 2>(p, max_m_tiles, s);
             if (waves == 4) return launch_gemm_pipe<FMT, EPI, 256, 2, 2, 2>(p, max_m_tiles, s);
@@ -1216,6 +1205,29 @@ int dispatch_tile(const GemmParams& p, TileChoice t, uint32_t max_m_tiles, hipSt
     return CMX_EINVAL;
 }
 
+// Pre-tiled weights (cmx_mx_pretile_weights): only the weights-to-registers kernel reads that order, so a problem it
+// cannot take is an error, not a reason to fall back.
+int check_pretiled(const GemmParams& p, int fmt, bool swiglu) {
+    CMX_REQUIRE(fmt == CMX_FMT_E4M3 || fmt == CMX_FMT_E5M2, "pre-tiled weights: 8-bit element formats only");
+    CMX_REQUIRE(p.kbytes % (4 * kSlabBytes) == 0, "pre-tiled weights: k must be a multiple of 512");
+    CMX_REQUIRE(p.scale_vec16, "pre-tiled weights: scale rows of both operands must be 16-byte aligned");
+    // (with the bf16 activation output on top, the SwiGLU epilogue no longer fits the register file beside the weight ring)
+    CMX_REQUIRE(!swiglu || p.act_bf16 == nullptr, "pre-tiled weights: no bf16 activation output (act_bf16 must be NULL)");
+    CMX_REQUIRE(swiglu || (p.out_type != CMX_OUT_FP32 && p.n % 8 == 0 && p.ldc % 8 == 0 && (reinterpret_cast<uintptr_t>(p.c) & 15u) == 0),
+                "pre-tiled weights: 16-bit output, n and ldc multiples of 8, c 16-byte aligned");
+    return CMX_OK;
+}
+
+int launch_pretiled(const GemmParams& p, int fmt, bool swiglu, uint32_t max_m_tiles, hipStream_t s) {
+    if (swiglu) return launch_gemm_wreg<CMX_FMT_E4M3, kEpiSwigluQuant>(p, max_m_tiles, s);
+    if (fmt == CMX_FMT_E4M3) {
+        if (p.out_type == CMX_OUT_BF16) return launch_gemm_wreg<CMX_FMT_E4M3, kEpiStoreBf16>(p, max_m_tiles, s);
+        return launch_gemm_wreg<CMX_FMT_E4M3, kEpiStoreFp16>(p, max_m_tiles, s);
+    }
+    if (p.out_type == CMX_OUT_BF16) return launch_gemm_wreg<CMX_FMT_E5M2, kEpiStoreBf16>(p, max_m_tiles, s);
+    return launch_gemm_wreg<CMX_FMT_E5M2, kEpiStoreFp16>(p, max_m_tiles, s);
+}
+
 int check_operands(const void* a, uint32_t lda, const void* as, uint32_t ld_as, const void* w, uint32_t ldw,
                    const void* ws, uint32_t ld_ws, uint32_t k, int fmt) {
     CMX_REQUIRE(a && as && w && ws, "null pointer");
@@ -1245,11 +1257,6 @@ bool scales_dword_aligned(const void* as, uint32_t ld_as, const void* ws, uint32
 #ifdef CMX_TEST_HOOKS
 extern "C" int cmx_debug_disable_streaming(int off) {
     cmx::g_disable_dl = off != 0;
-    return CMX_OK;
-}
-
-extern "C" int cmx_debug_w_pretiled(int on) {
-    cmx::g_w_pretiled = on;
     return CMX_OK;
 }
 
@@ -1303,29 +1310,27 @@ int gmm_common(GemmParams& p, const int32_t* group_sizes, uint32_t groups, uint3
     CMX_REQUIRE((uint64_t)p.n * p.ldw < (1ull << 32) && (uint64_t)p.lda * 256 < (1ull << 32),
                 "operand tile exceeds 32-bit offsets");
     CMX_REQUIRE((reinterpret_cast<uintptr_t>(workspace) & 3u) == 0, "workspace must be 4-byte aligned");
+    if (p.w_pretiled)
+        if (int rc = check_pretiled(p, fmt, swiglu); rc != CMX_OK) return rc;
     // average rows per group steers the tile height
     TileChoice t = choose_tile(ceil_div(m_total, groups), p.n, fmt, true);
+    if (p.w_pretiled) t = {256, 256, 5};     // the weights-to-registers kernel: 256 x 256 tiles, drawn from the counters
     int32_t* row_off = static_cast<int32_t*>(workspace);
     int32_t* tile_pref = row_off + (groups + 1);
     int32_t* tile_ctr = tile_pref + (groups + 1);
     hipLaunchKernelGGL(gmm_prepare_kernel, dim3(1), dim3(256), 0, s, group_sizes, groups, (uint32_t)t.tm, m_total, row_off,
                        tile_pref, tile_ctr);
     CMX_LAUNCH_CHECK();
-#ifdef CMX_TEST_HOOKS
-    p.w_pretiled = g_w_pretiled & 1;
-#endif
     p.row_off = row_off;
     p.tile_pref = tile_pref;
     // The persistent kernels draw their next tile from a per-XCD counter when tiles differ in cost (4 x 1 wavefronts skip
     // the MFMAs of absent rows).  With 2 x 2 wavefronts every tile costs the same, so those kernels walk their XCD's run in
     // fixed strides instead: no atomic whose result has to be waited for with everything else in flight.
     p.tile_ctr = t.waves == 4 ? nullptr : tile_ctr;
-#ifdef CMX_TEST_HOOKS
-    if (g_w_pretiled & 2) p.tile_ctr = nullptr;
-#endif
     p.groups = groups;
     p.w_tiles = swiglu ? ceil_div(p.n / 2, t.tw / 2) : ceil_div(p.n, t.tw);
     const uint32_t max_m_tiles = m_total / t.tm + groups;
+    if (p.w_pretiled) return launch_pretiled(p, fmt, swiglu, max_m_tiles, s);
     if (swiglu && p.act_bf16 != nullptr) return dispatch_tile<CMX_FMT_E4M3, kEpiSwigluQuantAct>(p, t, max_m_tiles, s);
     if (swiglu) return dispatch_tile<CMX_FMT_E4M3, kEpiSwigluQuant>(p, t, max_m_tiles, s);
     switch (fmt) {
@@ -1337,11 +1342,11 @@ int gmm_common(GemmParams& p, const int32_t* group_sizes, uint32_t groups, uint3
 }  // namespace
 }  // namespace cmx
 
-extern "C" int cmx_mx_gmm(const uint8_t* a, uint32_t lda, const uint8_t* a_scale, uint32_t ld_as, const uint8_t* b,
-                          const uint8_t* b_scale, void* c, uint32_t ldc, const int32_t* group_sizes, uint32_t groups,
-                          uint32_t m_total, uint32_t n, uint32_t k, int fmt, int out_type, void* workspace,
-                          cmx_stream_t stream) {
-    using namespace cmx;
+namespace cmx {
+namespace {
+int gmm_store(const uint8_t* a, uint32_t lda, const uint8_t* a_scale, uint32_t ld_as, const uint8_t* b, const uint8_t* b_scale,
+              void* c, uint32_t ldc, const int32_t* group_sizes, uint32_t groups, uint32_t m_total, uint32_t n, uint32_t k,
+              int fmt, int out_type, void* workspace, bool pretiled, cmx_stream_t stream) {
     if (m_total == 0 || n == 0) return CMX_OK;
     const uint32_t kbytes = fmt == CMX_FMT_E2M1 ? k / 2 : k;
     // weight scale rows are as every producer writes them: padded to an even count (the quantizer, the
@@ -1357,7 +1362,26 @@ extern "C" int cmx_mx_gmm(const uint8_t* a, uint32_t lda, const uint8_t* a_scale
     p.m = m_total; p.n = n; p.kbytes = kbytes; p.kblocks = k / 32; p.out_type = out_type;
     p.scale_vec = scales_dword_aligned(a_scale, ld_as, b_scale, ld_ws);
     p.scale_vec16 = scales_aligned16(a_scale, ld_as, b_scale, ld_ws);
+    p.w_pretiled = pretiled ? 1 : 0;
     return gmm_common(p, group_sizes, groups, m_total, workspace, fmt, false, static_cast<hipStream_t>(stream));
+}
+}  // namespace
+}  // namespace cmx
+
+extern "C" int cmx_mx_gmm(const uint8_t* a, uint32_t lda, const uint8_t* a_scale, uint32_t ld_as, const uint8_t* b,
+                          const uint8_t* b_scale, void* c, uint32_t ldc, const int32_t* group_sizes, uint32_t groups,
+                          uint32_t m_total, uint32_t n, uint32_t k, int fmt, int out_type, void* workspace,
+                          cmx_stream_t stream) {
+    return cmx::gmm_store(a, lda, a_scale, ld_as, b, b_scale, c, ldc, group_sizes, groups, m_total, n, k, fmt, out_type,
+                          workspace, false, stream);
+}
+
+extern "C" int cmx_mx_gmm_pretiled(const uint8_t* a, uint32_t lda, const uint8_t* a_scale, uint32_t ld_as,
+                                   const uint8_t* b_tiled, const uint8_t* b_scale, void* c, uint32_t ldc,
+                                   const int32_t* group_sizes, uint32_t groups, uint32_t m_total, uint32_t n, uint32_t k,
+                                   int fmt, int out_type, void* workspace, cmx_stream_t stream) {
+    return cmx::gmm_store(a, lda, a_scale, ld_as, b_tiled, b_scale, c, ldc, group_sizes, groups, m_total, n, k, fmt,
+                          out_type, workspace, true, stream);
 }
 
 extern "C" size_t cmx_int8_gmm_workspace_bytes(uint32_t groups, uint32_t n, uint32_t k, int trans_b) {
@@ -1423,7 +1447,7 @@ namespace {
 int gmm_swiglu_quant(const uint8_t* a, uint32_t lda, const uint8_t* a_scale, uint32_t ld_as, const uint8_t* b,
                      const uint8_t* b_scale, uint8_t* act_codes, uint32_t ld_act, uint8_t* act_scales, uint32_t ld_acts,
                      void* act_bf16, const int32_t* group_sizes, uint32_t groups, uint32_t m_total, uint32_t n, uint32_t k,
-                     void* workspace, cmx_stream_t stream) {
+                     void* workspace, bool pretiled, cmx_stream_t stream) {
     const uint32_t ld_ws = scale_cols(k);      // even-padded weight scale rows, as in cmx_mx_gmm
     int rc = check_operands(a, lda, a_scale, ld_as, b, k, b_scale, ld_ws, k, CMX_FMT_E4M3);
     if (rc != CMX_OK) return rc;
@@ -1440,6 +1464,7 @@ int gmm_swiglu_quant(const uint8_t* a, uint32_t lda, const uint8_t* a_scale, uin
     p.m = m_total; p.n = n; p.kbytes = k; p.kblocks = k / 32; p.out_type = CMX_OUT_BF16;
     p.scale_vec = scales_dword_aligned(a_scale, ld_as, b_scale, ld_ws);
     p.scale_vec16 = scales_aligned16(a_scale, ld_as, b_scale, ld_ws);
+    p.w_pretiled = pretiled ? 1 : 0;
     return gmm_common(p, group_sizes, groups, m_total, workspace, CMX_FMT_E4M3, true, static_cast<hipStream_t>(stream));
 }
 
@@ -1475,7 +1500,17 @@ extern "C" int cmx_mx_gmm_swiglu_quant(const uint8_t* a, uint32_t lda, const uin
                                        uint32_t k, void* workspace, cmx_stream_t stream) {
     if (m_total == 0 || n == 0) return CMX_OK;
     return cmx::gmm_swiglu_quant(a, lda, a_scale, ld_as, b, b_scale, act_codes, ld_act, act_scales, ld_acts, act_bf16,
-                                 group_sizes, groups, m_total, n, k, workspace, stream);
+                                 group_sizes, groups, m_total, n, k, workspace, false, stream);
+}
+
+extern "C" int cmx_mx_gmm_swiglu_quant_pretiled(const uint8_t* a, uint32_t lda, const uint8_t* a_scale, uint32_t ld_as,
+                                                const uint8_t* b_tiled, const uint8_t* b_scale, uint8_t* act_codes,
+                                                uint32_t ld_act, uint8_t* act_scales, uint32_t ld_acts, void* act_bf16,
+                                                const int32_t* group_sizes, uint32_t groups, uint32_t m_total,
+                                                uint32_t n, uint32_t k, void* workspace, cmx_stream_t stream) {
+    if (m_total == 0 || n == 0) return CMX_OK;
+    return cmx::gmm_swiglu_quant(a, lda, a_scale, ld_as, b_tiled, b_scale, act_codes, ld_act, act_scales, ld_acts,
+                                 act_bf16, group_sizes, groups, m_total, n, k, workspace, true, stream);
 }
 
 extern "C" uint32_t cmx_mx_gmm_noalloc_max_groups(void) { return cmx::kStaticGroups; }
@@ -1493,7 +1528,7 @@ extern "C" int cmx_mx_gmm_swiglu_quant_noalloc(const uint8_t* a, uint32_t lda, c
     // gmm_prepare_kernel rewrites every word of the metadata that the matmul kernel reads (and zeroes the tile
     // counters), so nothing of an earlier call survives into this one
     return gmm_swiglu_quant(a, lda, a_scale, ld_as, b, b_scale, act_codes, ld_act, act_scales, ld_acts, act_bf16,
-                            group_sizes, groups, m_total, n, k, meta, stream);
+                            group_sizes, groups, m_total, n, k, meta, false, stream);
 }
 
 // One-time set-up on the current device: raises the dynamic-LDS limit of every matmul kernel, has the runtime load the

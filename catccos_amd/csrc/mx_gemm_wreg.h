@@ -7,9 +7,9 @@
 // load.  The register file is the larger memory (512 KiB per CU against 160 KiB), and in the 4 x 1 wavefront layout the
 // 64 weight rows of a wavefront are read by that wavefront alone.  So here
 //   * each wavefront loads its own weight fragments straight into registers (buffer_load_dwordx4, the lane that
-//     feeds a row to the MFMA fetches that row's bytes), into a ring of FOUR slabs (128 VGPRs): the loads of slab
-//     s + 3 are issued while slab s is being multiplied and have two and a half slab times to land, with up to three
-//     slabs (96 KiB per CU) in flight;
+//     feeds a row to the MFMA fetches that row's bytes; the weights are stored pre-tiled so that such a load reads
+//     whole cache lines), into a ring of FOUR slabs (128 VGPRs): the loads of slab s + 3 are issued while slab s is
+//     being multiplied and have two and a half slab times to land, with up to three slabs (96 KiB per CU) in flight;
 //   * only the activation rows, which all four wavefronts read, go through the LDS (LDS-DMA into a ring of four
 //     32 KiB slots, three slabs ahead as well), together with the scale blocks of both operands;
 //   * the eight activation fragments of a step are refreshed in place: fragment j of the next step is read as soon
@@ -28,40 +28,36 @@
 //            scale block, two loads)
 //   step 1:  8 pairs; behind pair j the scale read and the two reads of fragment j of slab s + 1 (pair 0: also the two
 //            weight scales) and weight load j of slab s + 3
-// Scales need no byte shift here: a step multiplies the slab's 32-blocks (h, 2 + h) instead of (2h, 2h + 1) -- any
-// assignment of K positions to steps serves, as long as both operands use the same -- so the lanes of half-wave lh,
-// whose scale byte applies to the first (lh = 0) or second (lh = 1) block of an MFMA, find their bytes for step 0 and
-// step 1 side by side at byte 2 lh of the slab's dword: one ds_read_u16 per fragment, byte select 0 or 1 in the MFMA,
-// and the activation scale of fragment j is refreshed in place like the fragment itself.
+// The K positions are multiplied and summed in the order of the two-slot kernels (step h of a slab takes its 32-blocks
+// 2h and 2h + 1), so the results are the same bits.  The lanes of half-wave
+// lh, whose scale byte applies to the first (lh = 0) or second (lh = 1) block of an MFMA, need bytes lh (step 0) and
+// 2 + lh (step 1) of the slab's dword: the dword is read whole, shifted right by one byte in the upper half-wave right
+// before its first use (one VALU instruction), and the MFMAs select bytes 0 and 2.  The activation scale of fragment j
+// is refreshed in place like the fragment itself.  (Measured alternatives at 256 groups of ~256 rows, K = 7168: reading
+// the dword at byte address lh, which the LDS allows, +5 % kernel time over no shift at all; the shift under a half EXEC
+// mask +4 %; this shift +2.5 %; pairing the blocks (h, 2 + h), which needs no shift but sums K in another order than the
+// other kernels and so differs from them in the last bit of one output in a million, +0.)
 // The kernel is persistent like the two-slot grouped kernels: one workgroup per CU draws tiles from its XCD's counter,
 // and the load streams run on into the next tile while the last slabs of a tile are multiplied.
 #pragma once
 
 template <int IMM>
 __device__ __forceinline__ v4i wreg_load_b128(uint32_t voff, v4i rsrc, uint32_t soff) {
+    static_assert(IMM >= 0 && IMM < 4096, "immediate offset of a buffer load: twelve bits");
     v4i r;
     soff = __builtin_amdgcn_readfirstlane(soff);
-#if defined(CMX_WREG_WPOL) && CMX_WREG_WPOL == 1
-#define CMX_WREG_WPOLICY " nt"
-#elif defined(CMX_WREG_WPOL) && CMX_WREG_WPOL == 2
-#define CMX_WREG_WPOLICY " sc1 nt"
-#elif defined(CMX_WREG_WPOL) && CMX_WREG_WPOL == 3
-#define CMX_WREG_WPOLICY " sc0 sc1"
-#else
-#define CMX_WREG_WPOLICY ""
-#endif
-    asm volatile("buffer_load_dwordx4 %0, %1, %2, %3 offen offset:%4" CMX_WREG_WPOLICY : "=v"(r) : "v"(voff), "s"(rsrc), "s"(soff), "n"(IMM) : "memory");
+    asm volatile("buffer_load_dwordx4 %0, %1, %2, %3 offen offset:%4" : "=v"(r) : "v"(voff), "s"(rsrc), "s"(soff), "n"(IMM) : "memory");
     return r;
 }
 
-template <int OFF>
-__device__ __forceinline__ uint32_t lds_read_u16(uint32_t addr) {
-    uint32_t r;
-    asm volatile("ds_read_u16 %0, %1 offset:%2" : "=v"(r) : "v"(addr), "n"(OFF) : "memory");
-    return r;
+// r >>= sh (sh = 8 in lanes 32..63, 0 in the others): the scale dword of a slab holds the bytes of its four 32-blocks in
+// order; after this the lanes of either half-wave find their byte for step 0 (block lh) at byte 0 and that for step 1
+// (block 2 + lh) at byte 2
+__device__ __forceinline__ void shift_scale(uint32_t& r, uint32_t sh) {
+    asm volatile("v_lshrrev_b32 %0, %1, %0" : "+v"(r) : "v"(sh));
 }
 
-// acc += W-fragment x A-fragment with scale byte BYTE (0 or 1) of both scale registers; BIT as in mfma_acc
+// acc += W-fragment x A-fragment with scale byte BYTE (0 or 2) of both scale registers; BIT as in mfma_acc
 #define CMX_WREG_MFMA(SELTXT, EXTRA)                                                                            \
     if constexpr (BIT < 0)                                                                                      \
         asm volatile("v_mfma_scale_f32_32x32x64_f8f6f4 %0, %1, %2, %0, %3, %4 " SELTXT EXTRA                    \
@@ -73,50 +69,56 @@ __device__ __forceinline__ uint32_t lds_read_u16(uint32_t addr) {
                      : "+a"(acc) : "v"(w), "v"(a), "v"(sw), "v"(sa), "s"(live), "n"(BIT < 0 ? 0 : BIT) : "scc")
 template <int FMT, int BYTE, int BIT>
 __device__ __forceinline__ void mfma_acc_b01(v16f& acc, const v8i& w, const v8i& a, uint32_t sw, uint32_t sa, uint32_t live) {
-    static_assert(BYTE == 0 || BYTE == 1, "scale byte");
+    static_assert(BYTE == 0 || BYTE == 2, "scale byte");
     live = __builtin_amdgcn_readfirstlane(live);
-#ifdef CMX_WREG_NO_MFMA
-    asm volatile("" : "+a"(acc) : "v"(w), "v"(a), "v"(sw), "v"(sa), "s"(live));
-    return;
-#endif
     if constexpr (FMT == CMX_FMT_E4M3) {
-        if constexpr (BYTE == 0) { CMX_WREG_MFMA("op_sel_hi:[0,0,0]", ""); } else { CMX_WREG_MFMA("op_sel:[1,1,0] op_sel_hi:[0,0,0]", ""); }
+        if constexpr (BYTE == 0) { CMX_WREG_MFMA("op_sel_hi:[0,0,0]", ""); } else { CMX_WREG_MFMA("op_sel_hi:[1,1,0]", ""); }
     } else {
-        if constexpr (BYTE == 0) { CMX_WREG_MFMA("op_sel_hi:[0,0,0]", " cbsz:1 blgp:1"); } else { CMX_WREG_MFMA("op_sel:[1,1,0] op_sel_hi:[0,0,0]", " cbsz:1 blgp:1"); }
+        if constexpr (BYTE == 0) { CMX_WREG_MFMA("op_sel_hi:[0,0,0]", " cbsz:1 blgp:1"); } else { CMX_WREG_MFMA("op_sel_hi:[1,1,0]", " cbsz:1 blgp:1"); }
     }
 }
 #undef CMX_WREG_MFMA
+
+// LDS footprint: activation ring (four slots of 256 rows), ring of two scale blocks (16 bytes per row of both operands),
+// next-tile mailbox
+constexpr size_t kWregLdsBytes = (size_t)4 * 256 * 128 + (size_t)2 * 512 * 16 + 512;
 
 // LDS operations issued behind MFMA pair p of a step of kind K (0: first half of a slab, 1: second half): two fragment
 // reads; in the second half preceded by the scale read of that fragment for the next slab, and behind pair 0 by the two
 // weight scale reads as well.
 __host__ __device__ constexpr int wreg_lds_ops(int kind, int p) { return kind == 0 ? 2 : (3 + (p == 0 ? 2 : 0)); }
-// lgkmcnt that guarantees fragments j and j + 1 of a step of kind K (and with them the scales read before them) have
-// landed, asked right before pair j (j even): LDS returns in order, so it is the number of operations issued after the
-// reads of fragment j + 1 -- the rest of the previous step (kind 1 - K) and pairs 0..j-1 of this one.
-__host__ __device__ constexpr int wreg_frag_wait(int kind, int j) {
+// lgkmcnt that guarantees fragment j of a step of kind K (and with it the scale read before it) has landed, asked right
+// before pair j: LDS returns in order, so it is the number of operations issued after the reads of fragment j -- the rest
+// of the previous step (kind 1 - K) and pairs 0..j-1 of this one.  The counter has four bits: a smaller count only asks for
+// older reads as well.
+__host__ __device__ constexpr int wreg_frag_wait(int kind, int j, int fm) {
     int n = 0;
-    for (int p = j + 2; p < 8; ++p) n += wreg_lds_ops(1 - kind, p);
+    for (int p = j + 1; p < fm; ++p) n += wreg_lds_ops(1 - kind, p);
     for (int p = 0; p < j; ++p) n += wreg_lds_ops(kind, p);
-    return n < 15 ? n : 15;                    // the counter has four bits: a smaller count only asks for older reads as well
+    return n < 15 ? n : 15;
 }
+// loads behind pair j when `total` loads are spread over `pairs` pairs: indices [first, first + count)
+__host__ __device__ constexpr int wreg_first_load(int total, int pairs, int j) { return total * j / pairs; }
 
-// PRE: the weights come pre-tiled (cmx_mx_pretile_weights): [group][weight tile][slab][wavefront][load 0..7][lane][16 bytes],
-// 32 KiB per slab and tile, so that a weight load of a wavefront reads 1 KiB of consecutive bytes (eight whole cache lines)
-// instead of 32 bytes from each of 32 rows.
-template <int FMT, int EPI, bool PRE>
+// The weights come pre-tiled (cmx_mx_pretile_weights): [group][weight tile][slab][weight wavefront][load 0..7][lane][16 bytes],
+// 256 x 128 bytes per slab and tile, so that a weight load of a wavefront reads 1 KiB of consecutive bytes (eight whole cache
+// lines); from row-major weights the same load takes 32 bytes from each of 32 rows, and that many more visits to the
+// vector cache made the kernel a quarter slower than the two-slot ones.
+template <int FMT, int EPI>
 __global__ __launch_bounds__(256) void mx_gemm_wreg_kernel(const GemmParams p) {
     static_assert(FMT == CMX_FMT_E4M3 || FMT == CMX_FMT_E5M2, "8-bit element formats only");
     static_assert(EPI != kEpiStore, "persistent kernel: SwiGLU or lean 16-bit store epilogue");
-    constexpr int TW = 256, TM = 256, NW = 4, WW = 4, WM = 1, FW = 2, FM = 8, NF = FW + FM;
+    constexpr int TW = 256, TM = 256, NW = 4, WW = 4, WM = 1, FW = 2;
+    constexpr int NA = TM / 32;                                // activation fragments of the tile
+    constexpr int FM = (NA + WM - 1) / WM;                     // ... of a wavefront (fragment j of wavefront-row wm is fragment j * WM + wm of the tile)
     constexpr int kRing = 4;                                   // slabs in the weight register ring = slots of the activation ring
-    constexpr int kSlotBytes = TM * kSlabBytes;                // 32 KiB
+    constexpr int kSlotBytes = TM * kSlabBytes;
     constexpr int kScaleBase = kRing * kSlotBytes;
     constexpr int kScaleRows = TW + TM;
-    constexpr int kScaleSlotBytes = kScaleRows * 16;           // one block: 16 bytes (the scales of four slabs) per row
-    constexpr int kScaleRingBytes = 2 * kScaleSlotBytes;
-    constexpr int kALoads = TM / (8 * NW);                     // LDS-DMA loads per wavefront and slab (8)
-    static_assert(kALoads == 8 && FM == 8, "one activation load and one weight load behind every MFMA pair");
+    constexpr int kALoads = TM / (8 * NW);                     // LDS-DMA loads per wavefront and slab
+    constexpr int kWLoads = 8;                                 // weight loads per wavefront and slab: 2 steps x 2 fragments x 2 register halves
+    constexpr int kSlabLoads = kALoads + kWLoads;
+    static_assert(WW * WM == NW && TW % (WW * 32) == 0 && TM % 32 == 0, "tile geometry");
 
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t*)smem;
@@ -124,19 +126,29 @@ __global__ __launch_bounds__(256) void mx_gemm_wreg_kernel(const GemmParams p) {
     const uint32_t tid = threadIdx.x;
     const uint32_t lane = tid & 63u;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const uint32_t ww = wave;
+    const uint32_t ww = wave % WW, wm = wave / WW;
     const uint32_t l32 = lane & 31u, lh = lane >> 5;
 
-    // ---- tile sequence of this workgroup (as in the two-slot persistent kernels) -----------------------------------
+    // ---- tile sequence of this workgroup ---------------------------------------------------------------------------
+    // Every XCD owns a contiguous run of tiles, handed out as tickets: the workgroups start with tickets 0 .. G - 1 (G =
+    // workgroups per XCD) and draw further ones from the XCD's counter (or walk in strides of G when there is none).
+    // Whole rounds of G tickets are one tile each.  The tiles that are left for a last, partly filled round (L of them) are
+    // cut along their activation rows into S = G / L (at most 4) tickets each, so that round keeps every workgroup busy
+    // for a fraction of a tile time instead of some for a whole one; a part is just a tile of TM / S rows, its sums are the
+    // same bits, and the parts of a tile run side by side on one weight panel.
     const uint32_t m_tiles_all = count_m_tiles<TM>(p);
     const uint32_t total_tiles = m_tiles_all * p.w_tiles;
     uint32_t run_count;
     const uint32_t run_first = xcd_run(total_tiles, blockIdx.x % kXcds, run_count);
-    const uint32_t run_end = run_first + run_count;
-    const uint32_t tile_stride = gridDim.x / kXcds;
-    uint32_t tile_id = run_first + blockIdx.x / kXcds;
-    if (tile_id >= run_end) return;
-
+    const uint32_t tile_stride = gridDim.x / kXcds;                       // G
+    const uint32_t full_tickets = run_count / tile_stride * tile_stride;
+    const uint32_t left_tiles = run_count - full_tickets;                 // L
+    constexpr uint32_t kMaxSplit = TM % 128 == 0 ? 4 : 1;                // parts of whole 32-row fragments
+    const uint32_t split = left_tiles == 0 ? 1u : (tile_stride / left_tiles < kMaxSplit ? (tile_stride / left_tiles ? tile_stride / left_tiles : 1u) : kMaxSplit);
+    const uint32_t split_pow2 = split >= 4 ? 4u : (split >= 2 ? 2u : 1u);
+    const uint32_t run_tickets = full_tickets + left_tiles * split_pow2;
+    uint32_t ticket = blockIdx.x / kXcds;
+    if (ticket >= run_tickets) return;
     auto make_rsrc = [](const uint8_t* q) -> v4i {
         const uint64_t v = reinterpret_cast<uint64_t>(q);
         v4i r;
@@ -146,14 +158,14 @@ __global__ __launch_bounds__(256) void mx_gemm_wreg_kernel(const GemmParams p) {
         r[3] = 0x00020000;
         return r;
     };
-    // tile row of weight fragment f of this wavefront (SwiGLU: the gate fragment, then its up partner 128 rows on)
+    // tile row of weight fragment f of this wavefront (SwiGLU: the gate fragment, then its up partner half a tile on)
     constexpr int kWRowsPerWave = epi_is_swiglu_quant(EPI) ? TW / 2 / WW : TW / WW;
 #define CMX_WREG_WOFF(f) ((epi_is_swiglu_quant(EPI) ? ((f) < FW / 2 ? (f) * 32 : TW / 2 + ((f) - FW / 2) * 32) : (f) * 32))
     const uint32_t w_row_base = ww * kWRowsPerWave;
 
     // descriptors of the tile whose slabs the load streams are requesting
-    v4i w_rs, a_rs, ws_rs, as_rs;
-    uint32_t woff[FW], sgoff_w, sgoff_a;
+    v4i w_rs, a_rs, s_rs[2];
+    uint32_t sgoff[2];
     uint32_t a_last = 0;                        // last valid activation row of that tile
     auto wrow_of = [&](const Tile& t, uint32_t r) -> uint32_t {
         uint32_t gr;
@@ -173,44 +185,60 @@ __global__ __launch_bounds__(256) void mx_gemm_wreg_kernel(const GemmParams p) {
         t.mt = __builtin_amdgcn_readfirstlane(t.mt); t.row0 = __builtin_amdgcn_readfirstlane(t.row0);
         t.rows_valid = __builtin_amdgcn_readfirstlane(t.rows_valid);
     };
-    // scale blocks: this wavefront fetches those of weight rows 64 * wave .. and of activation rows 64 * wave ..
+    // Scale blocks: the rows of both operands form one sequence (weight rows, then activation rows) that is fetched in
+    // loads of 64 rows, two per wavefront: loads `wave` and `wave + 4` (where there is no such load, the first again).
+    constexpr int kScaleLoads = (kScaleRows + 63) / 64;
+    constexpr int kScaleRowsPadded = kScaleLoads * 64;
+    constexpr int kScaleSlotBytesP = kScaleRowsPadded * 16;
+    const uint32_t sload[2] = {wave, wave + 4 < (uint32_t)kScaleLoads ? wave + 4 : wave};
     auto aim_scales_at = [&](const Tile& t) {
-        ws_rs = make_rsrc(p.w_scale + (size_t)t.g * p.n * p.ld_ws);
-        as_rs = make_rsrc(p.a_scale + (size_t)t.row0 * p.ld_as);
-        const uint32_t ar = 64 * wave + lane;
-        sgoff_w = wrow_of(t, 64 * wave + lane) * p.ld_ws;
-        sgoff_a = (ar < t.rows_valid ? ar : t.rows_valid - 1) * p.ld_as;
+        const v4i ws_rs = make_rsrc(p.w_scale + (size_t)t.g * p.n * p.ld_ws);
+        const v4i as_rs = make_rsrc(p.a_scale + (size_t)t.row0 * p.ld_as);
+#pragma unroll
+        for (int k = 0; k < 2; ++k) {
+            const uint32_t c = 64 * sload[k] + lane;
+            const bool is_w = 64 * sload[k] < (uint32_t)TW;              // uniform: TW is a multiple of 64
+            const uint32_t ar = c - TW < t.rows_valid ? c - TW : t.rows_valid - 1;
+            sgoff[k] = is_w ? wrow_of(t, c) * p.ld_ws : ar * p.ld_as;
+#pragma unroll
+            for (int q = 0; q < 4; ++q) s_rs[k][q] = is_w ? ws_rs[q] : as_rs[q];
+        }
     };
     auto aim_tiles_at = [&](const Tile& t) {
-#ifdef CMX_WREG_SAME_W
-        if constexpr (PRE) w_rs = make_rsrc(p.w);
-#else
-        if constexpr (PRE) w_rs = make_rsrc(p.w + ((size_t)t.g * p.w_tiles + t.wt) * ((size_t)p.kbytes * TW));
-#endif
-        else w_rs = make_rsrc(p.w + (size_t)t.g * p.n * p.ldw);
-#ifdef CMX_WREG_SAME_A
-        a_rs = make_rsrc(p.a);
-#else
+        w_rs = make_rsrc(p.w + ((size_t)t.g * p.w_tiles + t.wt) * ((size_t)p.kbytes * TW));
         a_rs = make_rsrc(p.a + (size_t)t.row0 * p.lda);
-#endif
-        // weight fragment f, lane l: row l % 32 of the fragment, bytes 16 * (l / 32) + {0, 32, 64, 96} of the slab
-#pragma unroll
-        for (int f = 0; f < FW; ++f) {
-            if constexpr (PRE) woff[f] = wave * 8192 + lane * 16 + f * 4096;         // pre-tiled: index = step, not fragment
-            else woff[f] = mul_lo_u32(wrow_of(t, w_row_base + CMX_WREG_WOFF(f) + l32), p.ldw) + lh * 16;
-        }
         a_last = __builtin_amdgcn_readfirstlane(t.rows_valid - 1);
     };
     // LDS-DMA load i of this wavefront fills activation rows (4 i + wave) * 8 .. + 8; lane q -> row + q / 8, LDS chunk
     // q % 8, and fetches the global chunk that the XOR swizzle maps there (rows past the edge re-read the last one).
     // The per-lane offset is worked out in front of each load (three full-rate instructions) instead of being kept in
-    // eight registers: row = min(first row + 32 i, last valid row), offset = row * pitch + 16 * chunk.
+    // registers: row = min(first row + 32 i, last valid row), offset = row * pitch + 16 * chunk.
     const uint32_t a_row0 = wave * 8 + (lane >> 3);
+    // weight load j = (step, fragment, register half) of a slab: 1 KiB at j * 1024 of this wavefront's 8 KiB of the slab
+    // (one offset register per step: the immediate offset of a buffer load has twelve bits)
+    const uint32_t woff[2] = {ww * 8192 + lane * 16, ww * 8192 + lane * 16 + 4096};
     const uint32_t a_chunk16 = swz(a_row0, lane & 7u) * 16;      // (row & 15) does not depend on i
     const uint32_t a_lda = __builtin_amdgcn_readfirstlane(p.lda);
+    // ticket -> tile (whole, or one part of a tile of the last round); false when the part holds no rows
+    auto decode_ticket = [&](uint32_t t, Tile& out, uint32_t g_from) -> bool {
+        const bool whole = t < full_tickets;
+        const uint32_t tile = run_first + (whole ? t : full_tickets + (t - full_tickets) / split_pow2);
+        decode_tile<TM>(p, m_tiles_all, tile, out, g_from);
+        if (!whole && split_pow2 > 1) {
+            const uint32_t part = (t - full_tickets) % split_pow2, rpp = TM / split_pow2;
+            const uint32_t skip = part * rpp;
+            const uint32_t left = out.rows_valid > skip ? out.rows_valid - skip : 0u;
+            out.row0 += skip;
+            out.rows_valid = left < rpp ? left : rpp;
+        }
+        uniform_tile(out);
+        return out.rows_valid != 0;
+    };
     Tile tq;                                    // tile of the load streams
-    decode_tile<TM>(p, m_tiles_all, tile_id, tq, 0);
-    uniform_tile(tq);
+    while (!decode_ticket(ticket, tq, 0)) {     // (an empty part: on to this workgroup's next ticket)
+        ticket += tile_stride;                  // only tickets of the last round can be empty, and those have no successors in a strided walk
+        if (ticket >= run_tickets) return;
+    }
     aim_scales_at(tq);
     aim_tiles_at(tq);
     Tile tc = tq;                               // tile of the MFMA stream / epilogue
@@ -218,8 +246,8 @@ __global__ __launch_bounds__(256) void mx_gemm_wreg_kernel(const GemmParams p) {
     const uint32_t nslab = p.kbytes / kSlabBytes;            // a multiple of four (host check)
     const uint32_t nblk = nslab / 4;
     const uint32_t dma_base = __builtin_amdgcn_readfirstlane(lds0 + wave * 1024);
-    const uint32_t sdma_base_w = __builtin_amdgcn_readfirstlane(lds0 + kScaleBase + wave * 64 * 16);
-    const uint32_t sdma_base_a = __builtin_amdgcn_readfirstlane(lds0 + kScaleBase + (TW + wave * 64) * 16);
+    const uint32_t sdma_base[2] = {(uint32_t)__builtin_amdgcn_readfirstlane(lds0 + kScaleBase + sload[0] * 64 * 16),
+                                   (uint32_t)__builtin_amdgcn_readfirstlane(lds0 + kScaleBase + sload[1] * 64 * 16)};
     auto issue_a_load = [&](auto slot_c, auto i_c, uint32_t koff) {
         constexpr int slot = decltype(slot_c)::value, i = decltype(i_c)::value;
         (void)a_row0, (void)a_chunk16, (void)a_last;
@@ -232,26 +260,27 @@ __global__ __launch_bounds__(256) void mx_gemm_wreg_kernel(const GemmParams p) {
     auto issue_scale_block = [&](uint32_t byte_off) {
         const uint32_t pos = blocks_issued & 1u;
         ++blocks_issued;
-        dma_b128(sdma_base_w + pos * kScaleSlotBytes, sgoff_w, ws_rs, byte_off);
-        dma_b128(sdma_base_a + pos * kScaleSlotBytes, sgoff_a, as_rs, byte_off);
+        dma_b128(sdma_base[0] + pos * kScaleSlotBytesP, sgoff[0], s_rs[0], byte_off);
+        dma_b128(sdma_base[1] + pos * kScaleSlotBytesP, sgoff[1], s_rs[1], byte_off);
     };
 
     // ---- fragment and scale read addresses -----------------------------------------------------------------------
-    // a lane reads, for step h, the 16-byte chunks 2 h + lh (32-block h of the slab) and 4 + 2 h + lh (block 2 + h).  An
-    // LDS offset is a 16-bit immediate, so slots 0-1 and 2-3 need different base registers: one set of four, moved by
-    // 64 KiB twice per turn of four slabs
+    // a lane reads, for step h, the 16-byte chunks 4 h + lh (32-block 2h of the slab) and 4 h + 2 + lh (block 2h + 1) of its
+    // row.  One set of four base registers serves all slots: it points at the slot being read and is moved on between the
+    // two steps of a slab (the reads of step 1 already go to the next slab's slot); the immediate picks the fragment.
     const uint32_t x = (l32 & 7u) ^ ((l32 >> 3) & 1u);
     uint32_t ab[4];                             // [2 * step + half]
 #pragma unroll
-    for (int j = 0; j < 4; ++j) ab[j] = lds0 + l32 * kSlabBytes + ((2 * (j >> 1) + lh + 4 * (j & 1)) ^ x) * 16;
+    for (int j = 0; j < 4; ++j) ab[j] = lds0 + (wm * 32 + l32) * kSlabBytes + ((4 * (j >> 1) + 2 * (j & 1) + lh) ^ x) * 16;
     auto move_read_base = [&](int delta) {
         (void)ab;
 #pragma unroll
         for (int j = 0; j < 4; ++j) asm volatile("v_add_u32 %0, %1, %0" : "+v"(ab[j]) : "s"(delta));
     };
-    // scale bytes of this half-wave for the two steps of a slab: bytes 2 lh, 2 lh + 1 of the row's dword
-    const uint32_t swb = lds0 + kScaleBase + (w_row_base + l32) * 16 + 2 * lh;
-    const uint32_t sab = lds0 + kScaleBase + (TW + l32) * 16 + 2 * lh;
+    // scale dword of the row (the lanes of half-wave lh use its bytes lh and lh + 2: see shift_scale)
+    const uint32_t swb = lds0 + kScaleBase + (w_row_base + l32) * 16;
+    const uint32_t sab = lds0 + kScaleBase + (TW + wm * 32 + l32) * 16;
+    const uint32_t sshift = 8 * lh;
     uint32_t blocks_read = 0;                   // running count of the scale blocks whose first slab has been read
 
     v16f acc[FW][FM];
@@ -264,7 +293,7 @@ __global__ __launch_bounds__(256) void mx_gemm_wreg_kernel(const GemmParams p) {
 
     v4i wlo[kRing][2][FW], whi[kRing][2][FW];           // weight ring: [slab position][step][fragment], registers 0-3 / 4-7
     v4i alo[FM], ahi[FM];                               // the activation fragments of the step being multiplied (refreshed in place)
-    uint32_t sw[2][FW];                                 // weight scales of a slab (bytes 0, 1: steps 0, 1), by slab parity
+    uint32_t sw[2][FW];                                 // weight scales of a slab (bytes 0, 2: steps 0, 1), by slab parity
     uint32_t sa[FM];                                    // activation scales, refreshed in place like the fragments
 
     using I0 = std::integral_constant<int, 0>;
@@ -276,43 +305,49 @@ __global__ __launch_bounds__(256) void mx_gemm_wreg_kernel(const GemmParams p) {
         constexpr int h = i / 4, f = (i / 2) % 2, half = i % 2;
         (void)wlo, (void)whi, (void)woff;
         v4i& dst = half ? whi[pos][h][f] : wlo[pos][h][f];
-        if constexpr (PRE) dst = wreg_load_b128<(f * 2 + half) * 1024>(woff[h], w_rs, koff * TW);
-        else dst = wreg_load_b128<h * 32 + half * 64>(woff[f], w_rs, koff);
+        dst = wreg_load_b128<(f * 2 + half) * 1024>(woff[h], w_rs, koff * TW);
     };
-    // one 16-byte read of activation fragment fm for step `step` of the slab in slot `slot`
-    auto read_a_half = [&](auto slot_c, auto step_c, auto fm_c, auto half_c) {
-        constexpr int slot = decltype(slot_c)::value, step = decltype(step_c)::value, fm = decltype(fm_c)::value, half = decltype(half_c)::value;
+    // one 16-byte read of this wavefront's activation fragment j for step `step` from the slot the base registers point at
+    auto read_a_half = [&](auto step_c, auto j_c, auto half_c) {
+        constexpr int step = decltype(step_c)::value, j = decltype(j_c)::value, half = decltype(half_c)::value;
         (void)ab, (void)alo, (void)ahi;
-        v4i& dst = half ? ahi[fm] : alo[fm];
-        dst = lds_read_b128<(slot % 2) * kSlotBytes + fm * 32 * kSlabBytes>(ab[2 * step + half]);
+        v4i& dst = half ? ahi[j] : alo[j];
+        dst = lds_read_b128<j * WM * 32 * kSlabBytes>(ab[2 * step + half]);
     };
     auto read_w_scale_at = [&](uint32_t swb_at, auto set_c, auto f_c) {
         constexpr int set = decltype(set_c)::value, f = decltype(f_c)::value;
         (void)sw;
-        sw[set][f] = lds_read_u16<CMX_WREG_WOFF(f) * 16>(swb_at);
+        sw[set][f] = lds_read_b32<CMX_WREG_WOFF(f) * 16>(swb_at);
     };
-    auto read_a_scale_at = [&](uint32_t sab_at, auto fm_c) {
-        constexpr int fm = decltype(fm_c)::value;
+    auto read_a_scale_at = [&](uint32_t sab_at, auto j_c) {
+        constexpr int j = decltype(j_c)::value;
         (void)sa;
-        sa[fm] = lds_read_u16<fm * 32 * 16>(sab_at);
+        sa[j] = lds_read_b32<j * WM * 32 * 16>(sab_at);
     };
     // ring position and dword of the scales of the slab that follows the one at ring position P of the MFMA stream
     auto scale_read_offset = [&](int dword) -> uint32_t {
-        return __builtin_amdgcn_readfirstlane((blocks_read & 1u) * kScaleSlotBytes + dword * 4);
+        return __builtin_amdgcn_readfirstlane((blocks_read & 1u) * kScaleSlotBytesP + dword * 4);
     };
 
-    auto live_mask = [](uint32_t rows_valid) -> uint32_t { return __builtin_amdgcn_readfirstlane((1u << ((rows_valid + 31) / 32)) - 1u); };
-    uint32_t live = live_mask(tc.rows_valid);      // bit fm: activation block fm of the tile holds valid rows
+    // bit j: this wavefront's activation fragment j (fragment j * WM + wm of the tile) holds valid rows
+    auto live_mask = [&](uint32_t rows_valid) -> uint32_t {
+        const uint32_t frags = (rows_valid + 31) / 32;
+        uint32_t m = 0;
+#pragma unroll
+        for (int j = 0; j < FM; ++j) m |= ((uint32_t)j * WM + wm < frags ? 1u : 0u) << j;
+        return __builtin_amdgcn_readfirstlane(m);
+    };
+    uint32_t live = live_mask(tc.rows_valid);
 
     // ---- prologue: scale block 0, slabs 0..2 (activations before weights within a slab), fragments and scales of slab 0
     issue_scale_block(0);
     static_for<0, 3>([&](auto sc_) {
         constexpr int s = decltype(sc_)::value;
         static_for<0, kALoads>([&](auto ic) { issue_a_load(sc_, ic, s * kSlabBytes); });
-        static_for<0, 8>([&](auto ic) { issue_w_load(sc_, ic, s * kSlabBytes); });
+        static_for<0, kWLoads>([&](auto ic) { issue_w_load(sc_, ic, s * kSlabBytes); });
     });
-    asm volatile("s_waitcnt vmcnt(40)\n\ts_barrier" ::: "memory");          // scale block 0 and the activations of slab 0 are in
-    static_for<0, FM>([&](auto fc) { read_a_half(I0{}, I0{}, fc, I0{}); read_a_half(I0{}, I0{}, fc, I1{}); });
+    asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(kWLoads + 2 * kSlabLoads) : "memory");      // scale block 0 and the activations of slab 0 are in
+    static_for<0, FM>([&](auto fc) { read_a_half(I0{}, fc, I0{}); read_a_half(I0{}, fc, I1{}); });
     {
         const uint32_t off = scale_read_offset(0);
         static_for<0, FW>([&](auto fc) { read_w_scale_at(swb + off, I0{}, fc); });
@@ -321,9 +356,11 @@ __global__ __launch_bounds__(256) void mx_gemm_wreg_kernel(const GemmParams p) {
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
 
     auto fence_accumulators = [&]() {
-        v16f* const a = &acc[0][0];
-        asm volatile("s_nop 15\n\ts_nop 15" : "+a"(a[0]), "+a"(a[1]), "+a"(a[2]), "+a"(a[3]), "+a"(a[4]), "+a"(a[5]), "+a"(a[6]), "+a"(a[7]));
-        asm volatile("s_nop 15\n\ts_nop 15" : "+a"(a[8]), "+a"(a[9]), "+a"(a[10]), "+a"(a[11]), "+a"(a[12]), "+a"(a[13]), "+a"(a[14]), "+a"(a[15]));
+        static_for<0, FW * FM>([&](auto ic) {
+            constexpr int i = decltype(ic)::value;
+            (void)acc;
+            asm volatile("s_nop 15\n\ts_nop 15" : "+a"(acc[i / FM][i % FM]));
+        });
     };
     fence_accumulators();
 
@@ -332,16 +369,14 @@ __global__ __launch_bounds__(256) void mx_gemm_wreg_kernel(const GemmParams p) {
     // sblk: byte offset of the scale block issued at P = 0
     auto slab_body = [&](auto pos_c, uint32_t koff, uint32_t sblk) {
         constexpr int P = decltype(pos_c)::value;
-        constexpr int kNextSlot = (P + 1) % kRing, kLoadSlot = (P + 3) % kRing;
+        constexpr int kLoadSlot = (P + 3) % kRing;
         constexpr int kSet = P % 2, kNextSet = (P + 1) % 2;
-        using PosT = std::integral_constant<int, P>;
-        using NextSlotT = std::integral_constant<int, kNextSlot>;
         using LoadPosT = std::integral_constant<int, kLoadSlot>;
         using NextSetT = std::integral_constant<int, kNextSet>;
-        (void)acc, (void)sw, (void)sa, (void)wlo, (void)whi, (void)alo, (void)ahi, (void)live;
+        (void)acc, (void)sw, (void)sa, (void)wlo, (void)whi, (void)alo, (void)ahi, (void)live, (void)sshift;
         // own activation loads (and scale block) of slab s + 1 have landed: younger are the weights of slab s + 1 and all of
         // slab s + 2 (plus the scale block that went out with it when that was a position-0 slab)
-        asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(24 + (P == 1 ? 2 : 0)) : "memory");
+        asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(kWLoads + kSlabLoads + (P == 1 ? 2 : 0)) : "memory");
         // scales of the next slab: dword (P + 1) % 4 of its block; a new block starts with the slab at position 0
         if constexpr (P == 3) ++blocks_read;
         const uint32_t sc_off = scale_read_offset((P + 1) % 4);
@@ -349,40 +384,44 @@ __global__ __launch_bounds__(256) void mx_gemm_wreg_kernel(const GemmParams p) {
         // ---- step 0 ----
         static_for<0, FM>([&](auto jc) {
             constexpr int j = decltype(jc)::value;
-            if constexpr (j % 2 == 0) asm volatile("s_waitcnt lgkmcnt(%0)" ::"n"(wreg_frag_wait(0, j)) : "memory");
+            asm volatile("s_waitcnt lgkmcnt(%0)" ::"n"(wreg_frag_wait(0, j, FM)) : "memory");
+            // the scales of this slab were read as whole dwords (behind the pairs of the previous step): first use here
+            if constexpr (j == 0) {
+                shift_scale(sw[kSet][0], sshift);
+                shift_scale(sw[kSet][1], sshift);
+            }
+            shift_scale(sa[j], sshift);
             const v8i a = join8(alo[j], ahi[j]);
             mfma_acc_b01<FMT, 0, j>(acc[0][j], join8(wlo[P][0][0], whi[P][0][0]), a, sw[kSet][0], sa[j], live);
             mfma_acc_b01<FMT, 0, j>(acc[1][j], join8(wlo[P][0][1], whi[P][0][1]), a, sw[kSet][1], sa[j], live);
-            read_a_half(PosT{}, I1{}, jc, I0{});
-            read_a_half(PosT{}, I1{}, jc, I1{});
+            read_a_half(I1{}, jc, I0{});
+            read_a_half(I1{}, jc, I1{});
             if constexpr (P == 0 && j == 0) issue_scale_block(sblk);
-            issue_a_load(LoadPosT{}, jc, koff);
+            static_for<wreg_first_load(kALoads, FM, j), wreg_first_load(kALoads, FM, j + 1)>([&](auto ic) { issue_a_load(LoadPosT{}, ic, koff); });
         });
-        // the fragment reads of step 1 go to the next slab's slot: slots 0-1 and 2-3 have different base addresses
-        if constexpr (P == 1) move_read_base(2 * kSlotBytes);
-        if constexpr (P == 3) move_read_base(-2 * kSlotBytes);
+        // the fragment reads of step 1 go to the next slab's slot
+        move_read_base(P == 3 ? -3 * kSlotBytes : kSlotBytes);
         // ---- step 1 ----
         static_for<0, FM>([&](auto jc) {
             constexpr int j = decltype(jc)::value;
-            if constexpr (j % 2 == 0) asm volatile("s_waitcnt lgkmcnt(%0)" ::"n"(wreg_frag_wait(1, j)) : "memory");
+            asm volatile("s_waitcnt lgkmcnt(%0)" ::"n"(wreg_frag_wait(1, j, FM)) : "memory");
             const v8i a = join8(alo[j], ahi[j]);
-            mfma_acc_b01<FMT, 1, j>(acc[0][j], join8(wlo[P][1][0], whi[P][1][0]), a, sw[kSet][0], sa[j], live);
-            mfma_acc_b01<FMT, 1, j>(acc[1][j], join8(wlo[P][1][1], whi[P][1][1]), a, sw[kSet][1], sa[j], live);
+            mfma_acc_b01<FMT, 2, j>(acc[0][j], join8(wlo[P][1][0], whi[P][1][0]), a, sw[kSet][0], sa[j], live);
+            mfma_acc_b01<FMT, 2, j>(acc[1][j], join8(wlo[P][1][1], whi[P][1][1]), a, sw[kSet][1], sa[j], live);
             if constexpr (j == 0) {
                 read_w_scale_at(swb_at, NextSetT{}, I0{});
                 read_w_scale_at(swb_at, NextSetT{}, I1{});
             }
             read_a_scale_at(sab_at, jc);
-            read_a_half(NextSlotT{}, I0{}, jc, I0{});
-            read_a_half(NextSlotT{}, I0{}, jc, I1{});
-            issue_w_load(LoadPosT{}, jc, koff);
+            read_a_half(I0{}, jc, I0{});
+            read_a_half(I0{}, jc, I1{});
+            static_for<wreg_first_load(kWLoads, FM, j), wreg_first_load(kWLoads, FM, j + 1)>([&](auto ic) { issue_w_load(LoadPosT{}, ic, koff); });
         });
     };
 
     // ---- persistent loop: four slabs per turn, tiles change between turns ------------------------------------------
     uint32_t sm = 0;                 // first slab of the turn within the MFMA stream's tile
     bool next_ok = false;
-    uint32_t next_id = tile_id;
     Tile tn = tq;
     for (;;) {
         const bool last_turn = sm + 4 == nslab;
@@ -390,18 +429,24 @@ __global__ __launch_bounds__(256) void mx_gemm_wreg_kernel(const GemmParams p) {
         const uint32_t k0 = (sm + 3) * kSlabBytes;            // position 0 always requests a slab of the current tile
         if (last_turn) {
             // the load streams are about to run out of this tile: the next one (positions 1..3 and the scale block)
-            if (p.tile_ctr != nullptr) {
-                uint32_t* const mailbox = reinterpret_cast<uint32_t*>(smem + kScaleBase + kScaleRingBytes);
-                if (tid == 0) *mailbox = atomicAdd(reinterpret_cast<unsigned int*>(p.tile_ctr) + blockIdx.x % kXcds, 1u);
-                __syncthreads();
-                next_id = run_first + tile_stride + __builtin_amdgcn_readfirstlane(*mailbox);
-            } else {
-                next_id = tile_id + tile_stride;
+            next_ok = false;
+            for (;;) {
+                if (p.tile_ctr != nullptr) {
+                    uint32_t* const mailbox = reinterpret_cast<uint32_t*>(smem + kScaleBase + 2 * kScaleSlotBytesP);
+                    if (tid == 0) *mailbox = atomicAdd(reinterpret_cast<unsigned int*>(p.tile_ctr) + blockIdx.x % kXcds, 1u);
+                    __syncthreads();
+                    ticket = tile_stride + __builtin_amdgcn_readfirstlane(*mailbox);
+                    __syncthreads();                                     // everyone has read the mailbox before it is written again
+                } else {
+                    ticket += tile_stride;
+                }
+                if (ticket >= run_tickets) break;
+                if (decode_ticket(ticket, tn, tq.g)) {                   // tickets only grow, and with them the groups
+                    next_ok = true;
+                    break;
+                }
             }
-            next_ok = next_id < run_end;
             if (next_ok) {
-                decode_tile<TM>(p, m_tiles_all, next_id, tn, tq.g);      // tile ids only grow
-                uniform_tile(tn);
                 aim_scales_at(tn);
                 sblk = 0;
                 k1 = 0; k2 = kSlabBytes; k3 = 2 * kSlabBytes;
@@ -426,9 +471,8 @@ __global__ __launch_bounds__(256) void mx_gemm_wreg_kernel(const GemmParams p) {
             // the reads issued behind the last MFMAs target fragment registers that are dead on this path
             asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
             fence_accumulators();
-            epilogue<TW, TM, WW, WM, EPI, FW, FM>(p, tc, acc, ww, 0, lane);
+            epilogue<TW, TM, WW, WM, EPI, FW, FM>(p, tc, acc, ww, wm, lane);
             if (!next_ok) break;
-            tile_id = next_id;
             tc = tq;
             live = live_mask(tc.rows_valid);
             next_ok = false;
@@ -440,9 +484,9 @@ __global__ __launch_bounds__(256) void mx_gemm_wreg_kernel(const GemmParams p) {
 #pragma unroll
                     for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
             fence_accumulators();
-            // first fragments of the new tile again (slot 0 has landed and is visible; the scales of its slab 0 are
-            // already in their registers)
-            static_for<0, FM>([&](auto fc) { read_a_half(I0{}, I0{}, fc, I0{}); read_a_half(I0{}, I0{}, fc, I1{}); });
+            // first fragments of the new tile again (slot 0 has landed and is visible, and the base registers point at it;
+            // the scales of its slab 0 are already in their registers)
+            static_for<0, FM>([&](auto fc) { read_a_half(I0{}, fc, I0{}); read_a_half(I0{}, fc, I1{}); });
             asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
         }
     }

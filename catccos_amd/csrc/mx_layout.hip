@@ -437,3 +437,68 @@ extern "C" int cmx_mx_gmm_ex(const uint8_t* a, const uint8_t* a_scale, const uin
     const uint32_t kbytes = fmt == CMX_FMT_E2M1 ? k / 2 : k;
     return cmx_mx_gmm(a, kbytes, a_scale, k / 32, b, b_scale, c, ldc, group_sizes, groups, m_total, n, k, fmt, out_type, ws, stream);
 }
+
+// ---- pre-tiled weights -------------------------------------------------------------------------------------------
+// The weights-to-registers grouped kernel reads the weights of a 256-row tile slab by slab (128 bytes of K), and within
+// a slab every wavefront reads its own 8 KiB as eight loads of 1 KiB: [group][tile][slab][wavefront 0..3][step h]
+// [fragment f][register half][lane / 32][lane % 32][16 bytes].  The piece at (h, f, half, lh, l32) is bytes
+// 128 slab + 64 h + 32 half + 16 lh .. + 16 of the tile row that lane l32 feeds to the MFMA as weight fragment f:
+//   plain tiles    row 256 tile + 64 wavefront + 32 f + l32
+//   gate|up tiles  row 128 tile + 32 wavefront + l32 of the gate half (f = 0) or of the up half (f = 1)
+// (rows past the end repeat the last one, as the kernels' own clamped reads do).
+namespace cmx {
+namespace {
+constexpr uint32_t kPretileRows = 256;
+
+__global__ __launch_bounds__(512) void mx_pretile_weights_kernel(const uint8_t* __restrict__ src, uint8_t* __restrict__ dst,
+                                                                 uint32_t n, uint32_t kbytes, uint32_t w_tiles, int pair) {
+    // one workgroup: the 512 pieces of one (group, tile, slab, wavefront) -- 64 rows x 128 bytes, read as whole lines
+    const uint32_t t = threadIdx.x;
+    const uint32_t l32 = t & 31u, lh = (t >> 5) & 1u, half = (t >> 6) & 1u, f = (t >> 7) & 1u, h = t >> 8;
+    const uint32_t nslab = kbytes / 128;
+    const uint32_t ww = blockIdx.x & 3u;
+    const uint32_t slab = (blockIdx.x >> 2) % nslab;
+    const uint32_t tile = (blockIdx.x >> 2) / nslab;          // tile of the group
+    const uint32_t g = blockIdx.y;
+    uint32_t row;
+    if (pair) {
+        const uint32_t hn = n >> 1;
+        uint32_t r = tile * (kPretileRows / 2) + ww * 32 + l32;
+        r = r < hn ? r : hn - 1;
+        row = f ? hn + r : r;
+    } else {
+        row = tile * kPretileRows + ww * 64 + f * 32 + l32;
+        row = row < n ? row : n - 1;
+    }
+    const uint32_t col = slab * 128 + h * 64 + half * 32 + lh * 16;
+    const uint4 v = *reinterpret_cast<const uint4*>(src + ((size_t)g * n + row) * kbytes + col);
+    const size_t piece = (((size_t)g * w_tiles + tile) * nslab + slab) * 2048 + ww * 512 + t;
+    *reinterpret_cast<uint4*>(dst + piece * 16) = v;
+}
+
+uint32_t pretile_tiles(uint32_t n, int pair) { return pair ? ceil_div(n / 2, kPretileRows / 2) : ceil_div(n, kPretileRows); }
+}  // namespace
+}  // namespace cmx
+
+extern "C" size_t cmx_mx_pretiled_weight_bytes(uint32_t groups, uint32_t n, uint32_t k, int pair_gate_up) {
+    if (groups == 0 || n == 0 || k == 0 || k % 512 != 0 || (pair_gate_up && n % 64 != 0)) return 0;
+    return (size_t)groups * cmx::pretile_tiles(n, pair_gate_up) * cmx::kPretileRows * k;
+}
+
+extern "C" int cmx_mx_pretile_weights(const uint8_t* b, uint8_t* out, uint32_t groups, uint32_t n, uint32_t k,
+                                      int pair_gate_up, cmx_stream_t stream) {
+    using namespace cmx;
+    if (groups == 0 || n == 0) return CMX_OK;
+    CMX_REQUIRE(b && out, "null pointer");
+    CMX_REQUIRE(k > 0 && k % 512 == 0, "k must be a positive multiple of 512");
+    CMX_REQUIRE(!pair_gate_up || n % 64 == 0, "gate|up weights need n to be a multiple of 64");
+    CMX_REQUIRE(aligned16(b) && aligned16(out), "weights must be 16-byte aligned");
+    CMX_REQUIRE(groups <= 65535, "at most 65535 groups");
+    const uint32_t w_tiles = pretile_tiles(n, pair_gate_up);
+    const uint64_t blocks = (uint64_t)w_tiles * (k / 128) * 4;
+    CMX_REQUIRE(blocks < (1ull << 31), "weight matrix too large");
+    hipLaunchKernelGGL(mx_pretile_weights_kernel, dim3((uint32_t)blocks, groups), dim3(512), 0, static_cast<hipStream_t>(stream), b,
+                       out, n, k, w_tiles, pair_gate_up ? 1 : 0);
+    CMX_LAUNCH_CHECK();
+    return CMX_OK;
+}

@@ -162,26 +162,66 @@ def gmm_workspace(groups: int, device) -> torch.Tensor:
     return torch.empty(lib.cmx_mx_gmm_workspace_bytes(groups), dtype=torch.uint8, device=device)
 
 
+class PretiledWeights:
+    """Expert weights [groups, n, k] (8-bit codes) in the tiled order of cmx_mx_pretile_weights; ``pair_gate_up``
+    says which of the two grouped matmuls the tiling is for (True: mx_gmm_swiglu_quant, False: mx_gmm)."""
+
+    def __init__(self, data: torch.Tensor, groups: int, n: int, k: int, pair_gate_up: bool):
+        self.data, self.groups, self.n, self.k, self.pair_gate_up = data, groups, n, k, pair_gate_up
+
+    @property
+    def shape(self):
+        return (self.groups, self.n, self.k)
+
+
+def pretile_weights(b: torch.Tensor, pair_gate_up: bool) -> PretiledWeights:
+    """b u8 [G, n, k] dense -> PretiledWeights (one pass over the weights; meant for weight-load time)."""
+    _need_cuda(b)
+    assert b.dtype == torch.uint8 and b.dim() == 3 and b.is_contiguous()
+    g, n, k = b.shape
+    lib = _lib.load()
+    nbytes = lib.cmx_mx_pretiled_weight_bytes(g, n, k, int(pair_gate_up))
+    if nbytes == 0:
+        raise ValueError("pre-tiled weights need k % 512 == 0 (and n % 64 == 0 for gate|up weights)")
+    out = torch.empty(nbytes, dtype=torch.uint8, device=b.device)
+    _lib.check(lib.cmx_mx_pretile_weights(_p(b), _p(out), g, n, k, int(pair_gate_up), _stream()))
+    return PretiledWeights(out, g, n, k, bool(pair_gate_up))
+
+
+def _weights(b, pair_gate_up: bool):
+    """(pointer, pretiled?) of a weight argument: a dense tensor or PretiledWeights of the matching kind."""
+    if isinstance(b, PretiledWeights):
+        assert b.pair_gate_up == pair_gate_up, "weights were pre-tiled for the other grouped matmul"
+        return _p(b.data), True
+    assert b.is_contiguous()
+    return _p(b), False
+
+
 def mx_gmm(a, a_scale, b, b_scale, group_sizes, k: int, fmt: str = "E4M3", out: str = "bf16", c=None, workspace=None):
-    """a [m_total, k], b [G, n, k], group_sizes int32 [G] on device -> c [m_total, n] (rows past the groups untouched)."""
-    _need_cuda(a, a_scale, b, b_scale, group_sizes)
-    assert b.is_contiguous() and b_scale.is_contiguous() and group_sizes.dtype == torch.int32
+    """a [m_total, k], b [G, n, k] (dense tensor or PretiledWeights), group_sizes int32 [G] on device -> c [m_total, n]
+    (rows past the groups untouched)."""
+    _need_cuda(a, a_scale, b_scale, group_sizes)
+    assert b_scale.is_contiguous() and group_sizes.dtype == torch.int32
+    bp, tiled = _weights(b, False)
     m, (g, n) = a.shape[0], b.shape[:2]
     if c is None:
         c = torch.zeros((m, n), dtype=_OUT_DTYPE[out], device=a.device)
     if workspace is None:
         workspace = gmm_workspace(g, a.device)
     lib = _lib.load()
-    _lib.check(lib.cmx_mx_gmm(_p(a), a.stride(0), _p(a_scale), a_scale.stride(0), _p(b), _p(b_scale), _p(c), c.stride(0),
-                              _p(group_sizes), g, m, n, k, FMT[fmt], OUT[out], _p(workspace), _stream()))
+    fn = lib.cmx_mx_gmm_pretiled if tiled else lib.cmx_mx_gmm
+    _lib.check(fn(_p(a), a.stride(0), _p(a_scale), a_scale.stride(0), bp, _p(b_scale), _p(c), c.stride(0),
+                  _p(group_sizes), g, m, n, k, FMT[fmt], OUT[out], _p(workspace), _stream()))
     return c
 
 
 def mx_gmm_swiglu_quant(a, a_scale, b, b_scale, group_sizes, k: int, want_bf16: bool = False, workspace=None,
                         outs=None):
-    """GMM1 + SwiGLU + MX requant.  b [G, n, k] (gate rows then up rows).  Returns (codes [m, n/2], scales, act_bf16|None)."""
-    _need_cuda(a, a_scale, b, b_scale, group_sizes)
-    assert b.is_contiguous() and b_scale.is_contiguous() and group_sizes.dtype == torch.int32
+    """GMM1 + SwiGLU + MX requant.  b [G, n, k] (gate rows then up rows; dense tensor or PretiledWeights).
+    Returns (codes [m, n/2], scales, act_bf16|None)."""
+    _need_cuda(a, a_scale, b_scale, group_sizes)
+    assert b_scale.is_contiguous() and group_sizes.dtype == torch.int32
+    bp, tiled = _weights(b, True)
     m, (g, n) = a.shape[0], b.shape[:2]
     half = n // 2
     if outs is None:
@@ -193,9 +233,9 @@ def mx_gmm_swiglu_quant(a, a_scale, b, b_scale, group_sizes, k: int, want_bf16: 
     if workspace is None:
         workspace = gmm_workspace(g, a.device)
     lib = _lib.load()
-    _lib.check(lib.cmx_mx_gmm_swiglu_quant(_p(a), a.stride(0), _p(a_scale), a_scale.stride(0), _p(b), _p(b_scale),
-                                           _p(codes), codes.stride(0), _p(scales), scales.stride(0), _p(act),
-                                           _p(group_sizes), g, m, n, k, _p(workspace), _stream()))
+    fn = lib.cmx_mx_gmm_swiglu_quant_pretiled if tiled else lib.cmx_mx_gmm_swiglu_quant
+    _lib.check(fn(_p(a), a.stride(0), _p(a_scale), a_scale.stride(0), bp, _p(b_scale), _p(codes), codes.stride(0),
+                  _p(scales), scales.stride(0), _p(act), _p(group_sizes), g, m, n, k, _p(workspace), _stream()))
     return codes, scales, act
 
 
@@ -281,19 +321,29 @@ def ffn_workspace_layout(m: int, k: int, n: int, experts: int, top_k: int) -> di
 def dispatch_ffn_combine(x, expert_idx, gate_weight, w1, w1_scale, w2, w2_scale, workspace=None, out=None):
     """torch.ops.catccos.ascend950_dispatch_ffn_combine(x, expert_idx, gate_weight, w1, w1_scale, w2, w2_scale)
     on one GPU: x bf16 [m,k]; expert_idx int32 [m,topK]; gate_weight fp32 [m,topK];
-    w1 [E,n,k] + w1_scale [E,n,k/32]; w2 [E,k,n/2] + w2_scale [E,k,n/64] -> bf16 [m,k]."""
-    _need_cuda(x, expert_idx, gate_weight, w1, w1_scale, w2, w2_scale)
+    w1 [E,n,k] + w1_scale [E,n,k/32]; w2 [E,k,n/2] + w2_scale [E,k,n/64] -> bf16 [m,k].
+    w1 and w2 may both be PretiledWeights (w1 tiled with pair_gate_up=True, w2 with False): same result, through
+    cmx_dispatch_ffn_combine_pretiled."""
+    _need_cuda(x, expert_idx, gate_weight, w1_scale, w2_scale)
     m, k = x.shape
     e, n = w1.shape[:2]
     top_k = expert_idx.shape[1]
-    for t in (x, expert_idx, gate_weight, w1, w1_scale, w2, w2_scale):
+    for t in (x, expert_idx, gate_weight, w1_scale, w2_scale):
         assert t.is_contiguous()
+    w1p, tiled1 = _weights(w1, True)
+    w2p, tiled2 = _weights(w2, False)
+    assert tiled1 == tiled2, "pre-tile both weight tensors or neither"
     lib = _lib.load()
     if workspace is None:
         workspace = torch.empty(ffn_workspace_bytes(m, k, n, e, top_k), dtype=torch.uint8, device=x.device)
     if out is None:
         out = torch.empty((m, k), dtype=x.dtype, device=x.device)
+    if tiled1:
+        _lib.check(lib.cmx_dispatch_ffn_combine_pretiled(
+            _stream(), _p(x), _p(expert_idx), _p(gate_weight), w1p, _p(w1_scale), w2p, _p(w2_scale), _p(out),
+            _p(workspace), m, k, n, e, top_k))
+        return out
     _lib.check(lib.catccos_ascend950_dispatch_ffn_combine(
-        0, _stream(), 0, _p(x), _p(expert_idx), _p(gate_weight), _p(w1), _p(w1_scale), _p(w2), _p(w2_scale), _p(out),
+        0, _stream(), 0, _p(x), _p(expert_idx), _p(gate_weight), w1p, _p(w1_scale), w2p, _p(w2_scale), _p(out),
         _p(workspace), None, m, k, n, e, top_k, 1))
     return out

@@ -171,6 +171,44 @@ int cmx_mx_gmm_swiglu_quant_noalloc(const uint8_t* a, uint32_t lda, const uint8_
                                     uint32_t k, cmx_stream_t stream);
 
 /* ------------------------------------------------------------------------------------------
+ * Pre-tiled expert weights (8-bit element formats).  No counterpart in the reference's interface: its operators take
+ * the weights in the layout tag the caller names and the AIC block re-tiles them through L1 on every use
+ * (include/catccos/dgemm/kernel/ascend950_alltoall_gmm.hpp:193-323).  On this GPU a grouped matmul whose groups hold
+ * about one tile of rows streams every weight byte from HBM exactly once, and it does so fastest when each wavefront
+ * loads the fragments it multiplies straight into its registers; for that the bytes a wavefront loads together must lie
+ * together.  cmx_mx_pretile_weights rewrites dense [groups, n, k] codes ONCE (at weight-load time) into that order:
+ *   [group][256-row tile][128-byte K slab][wavefront 0..3][1 KiB load 0..7][lane 0..63][16 bytes]
+ * (cmx_mx_pretiled_weight_bytes bytes: groups * tiles * 256 * k, rows past n repeat the last row; 0 for shapes the
+ * format does not cover).  pair_gate_up = 1 tiles the weights of cmx_mx_gmm_swiglu_quant, whose tiles pair 128 gate
+ * rows with their 128 up rows; 0 those of cmx_mx_gmm.  The scales stay as they are ([groups, n, RoundUp2(k/32)]).
+ *
+ * cmx_mx_gmm_pretiled / cmx_mx_gmm_swiglu_quant_pretiled are cmx_mx_gmm / cmx_mx_gmm_swiglu_quant with b_tiled in
+ * place of b: same arguments otherwise, bit-identical results.  They need what the kernel behind them needs and fail
+ * with CMX_EINVAL (nothing launched) otherwise: E4M3 or E5M2, k a multiple of 512, scale rows of both operands
+ * 16-byte aligned (pointer and pitch); cmx_mx_gmm_pretiled also a 16-bit output type with n and ldc multiples of 8 and
+ * c 16-byte aligned; cmx_mx_gmm_swiglu_quant_pretiled act_bf16 == NULL (codes and scales only).  cmx_dispatch_ffn_combine_pretiled is catccos_ascend950_dispatch_ffn_combine (one device) on
+ * w1 tiled with pair_gate_up = 1 and w2 tiled with pair_gate_up = 0; K % 512 == 0 and N % 1024 == 0.
+ * Measured at 256 experts x 256 routed rows, K = 7168, N = 4096: GMM1 3 % and GMM2 8 % faster than on row-major
+ * weights; with 2048 rows per expert the row-major kernels are the faster ones (the weight stream is shared there).
+ * ---------------------------------------------------------------------------------------- */
+size_t cmx_mx_pretiled_weight_bytes(uint32_t groups, uint32_t n, uint32_t k, int pair_gate_up);
+int cmx_mx_pretile_weights(const uint8_t* b, uint8_t* b_tiled, uint32_t groups, uint32_t n, uint32_t k,
+                           int pair_gate_up, cmx_stream_t stream);
+int cmx_mx_gmm_pretiled(const uint8_t* a, uint32_t lda, const uint8_t* a_scale, uint32_t ld_as, const uint8_t* b_tiled,
+                        const uint8_t* b_scale, void* c, uint32_t ldc, const int32_t* group_sizes, uint32_t groups,
+                        uint32_t m_total, uint32_t n, uint32_t k, int fmt, int out_type, void* workspace,
+                        cmx_stream_t stream);
+int cmx_mx_gmm_swiglu_quant_pretiled(const uint8_t* a, uint32_t lda, const uint8_t* a_scale, uint32_t ld_as,
+                                     const uint8_t* b_tiled, const uint8_t* b_scale, uint8_t* act_codes,
+                                     uint32_t ld_act, uint8_t* act_scales, uint32_t ld_acts, void* act_bf16,
+                                     const int32_t* group_sizes, uint32_t groups, uint32_t m_total, uint32_t n,
+                                     uint32_t k, void* workspace, cmx_stream_t stream);
+int cmx_dispatch_ffn_combine_pretiled(cmx_stream_t stream, const uint8_t* x, const uint8_t* expertIdx,
+                                      const uint8_t* gateWeight, const uint8_t* w1_tiled, const uint8_t* w1Scale,
+                                      const uint8_t* w2_tiled, const uint8_t* w2Scale, uint8_t* out, uint8_t* workspace,
+                                      uint32_t m, uint32_t k, uint32_t n, uint32_t localExperts, uint32_t topK);
+
+/* ------------------------------------------------------------------------------------------
  * Operands stored with K as the slow axis.
  * The reference's generators write B either transposed ([N, K], what cmx_mx_gemm takes) or as
  * [K, N] codes with scales [K/64, N, 2] (examples/ascend950_mxfp8_matmul_reduce_scatter/scripts/

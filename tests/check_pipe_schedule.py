@@ -1,5 +1,5 @@
 #!/usr/bin/env python3
-"""Checks the compiled form of the hand-scheduled matmul kernels (mx_gemm_pipe.h, mx_gemm_pipe_fp4.h).
+"""Checks the compiled form of the hand-scheduled matmul kernels (mx_gemm_pipe.h, mx_gemm_pipe_fp4.h, mx_gemm_wreg.h).
 
 The instruction stream between a kernel's first and last MFMA is written out by hand, one instruction per asm
 statement; the compiler adds the address arithmetic around it and allocates the registers.  Two things it may also
@@ -40,7 +40,14 @@ FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-Xclang", "-target-featu
 # persistent 2 x 2 kernels send all 8 weight loads early -- plus 2 prefetch loads in the persistent 2 x 2 kernels)
 #   mx_gemm_pipe_kernel<FMT, EPI, TM, WW, WM, NSLOT>; EPI 0 store, 1 SwiGLU + requant, 2 lean bf16, 4 lean fp16, 5 = 1 + bf16 activations
 #   mx_gemm_pipe_fp4_kernel<EPI, WW, WM>
+#   mx_gemm_wreg_kernel<FMT, EPI>: the wait at the start of a slab leaves the weight loads of the next slab and all loads of the
+#   one after in flight (8 + 16), two more behind the slab that sent a scale block
 KERNELS = [
+    ("mx_gemm_wreg_kernel<0, 1>", {24, 26}),
+    ("mx_gemm_wreg_kernel<0, 2>", {24, 26}),
+    ("mx_gemm_wreg_kernel<0, 4>", {24, 26}),
+    ("mx_gemm_wreg_kernel<1, 2>", {24, 26}),
+    ("mx_gemm_wreg_kernel<1, 4>", {24, 26}),
     ("mx_gemm_pipe_kernel<0, 1, 256, 2, 2, 2>", {10}),
     ("mx_gemm_pipe_kernel<0, 1, 256, 4, 1, 2>", {8}),
     ("mx_gemm_pipe_kernel<0, 5, 256, 2, 2, 2>", {10}),          # SwiGLU + requant that also writes the bf16 activations

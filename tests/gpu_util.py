@@ -38,12 +38,11 @@ def close_bf16(out_bits, gold_f32, rtol=1e-2, atol=1e-2):
 import ctypes as _C
 import os as _os
 
-TEST_LIB_PATH = _os.environ.get("CMX_TEST_LIB") or _os.path.join(_os.path.dirname(_os.path.abspath(__file__)), "lib", "libcatccos_mx_test.so")
+TEST_LIB_PATH = _os.path.join(_os.path.dirname(_os.path.abspath(__file__)), "lib", "libcatccos_mx_test.so")
 _HOOKS = {
     "cmx_mfma_raw_probe": (_C.c_int, [_C.c_void_p] * 5 + [_C.c_int] * 3 + [_C.c_void_p]),
     "cmx_debug_force_tile": (_C.c_int, [_C.c_int] * 3),
     "cmx_debug_disable_streaming": (_C.c_int, [_C.c_int]),
-    "cmx_debug_w_pretiled": (_C.c_int, [_C.c_int]),
 }
 _test_lib = None
 

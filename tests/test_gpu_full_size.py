@@ -262,3 +262,10 @@ def test_config4_ffn_full_size():
     # doubling every gate weight doubles the bf16 output exactly (the combine multiplies, then adds in fp32)
     out2 = ops.dispatch_ffn_combine(x, idx, p * 2, w1, w1s, w2, w2s, workspace=ws)
     assert torch.equal(out2.float(), out.float() * 2)
+    # (5) the same chain on pre-tiled weights (the weights-to-registers kernel in both matmuls): same bits at every stage
+    w1t, w2t = ops.pretile_weights(w1, True), ops.pretile_weights(w2, False)
+    keep_codes, keep_scales, keep_y = act_codes.clone(), act_scales.clone(), y.clone()
+    ws.fill_(0x5A)
+    out_t = ops.dispatch_ffn_combine(x, idx, p, w1t, w1s, w2t, w2s, workspace=ws)
+    assert torch.equal(act_codes, keep_codes) and torch.equal(act_scales, keep_scales)
+    assert torch.equal(y, keep_y) and torch.equal(out_t, out)
