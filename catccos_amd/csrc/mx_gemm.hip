@@ -1064,9 +1064,10 @@ int launch_gemm_pipe(const GemmParams& p, uint32_t max_m_tiles, hipStream_t s) {
     return CMX_OK;
 }
 
-template <int FMT, int EPI>
+template <int FMT, int EPI, int TM>
 int launch_gemm_wreg(const GemmParams& p, uint32_t max_m_tiles, hipStream_t s) {
-    constexpr auto kfn = mx_gemm_wreg_kernel<FMT, EPI>;
+    constexpr auto kfn = mx_gemm_wreg_kernel<FMT, EPI, TM>;
+    constexpr size_t kWregLdsBytes = wreg_lds_bytes(TM);
     if (int rc = allow_dynamic_lds<kfn, kWregLdsBytes>(); rc != CMX_OK) return rc;
     const uint64_t tiles = (uint64_t)max_m_tiles * p.w_tiles;
     CMX_REQUIRE(tiles > 0 && tiles < (1ull << 31), "tile count out of range");
@@ -1126,8 +1127,10 @@ struct TileChoice {
 
 #ifdef CMX_TEST_HOOKS
 TileChoice g_force_tile = {0, 0, 0};   // tw == 0 -> heuristic
+int g_pretiled_tile_rows = 0;          // 0 -> heuristic
 #else
 constexpr TileChoice g_force_tile = {0, 0, 0};
+constexpr int g_pretiled_tile_rows = 0;
 #endif
 
 // waves: at 256 x 256 "4" and "5" select the hand-scheduled kernel in its 2 x 2 and 4 x 1 wavefront layouts
@@ -1218,14 +1221,15 @@ int check_pretiled(const GemmParams& p, int fmt, bool swiglu) {
     return CMX_OK;
 }
 
+template <int TM>
 int launch_pretiled(const GemmParams& p, int fmt, bool swiglu, uint32_t max_m_tiles, hipStream_t s) {
-    if (swiglu) return launch_gemm_wreg<CMX_FMT_E4M3, kEpiSwigluQuant>(p, max_m_tiles, s);
+    if (swiglu) return launch_gemm_wreg<CMX_FMT_E4M3, kEpiSwigluQuant, TM>(p, max_m_tiles, s);
     if (fmt == CMX_FMT_E4M3) {
-        if (p.out_type == CMX_OUT_BF16) return launch_gemm_wreg<CMX_FMT_E4M3, kEpiStoreBf16>(p, max_m_tiles, s);
-        return launch_gemm_wreg<CMX_FMT_E4M3, kEpiStoreFp16>(p, max_m_tiles, s);
+        if (p.out_type == CMX_OUT_BF16) return launch_gemm_wreg<CMX_FMT_E4M3, kEpiStoreBf16, TM>(p, max_m_tiles, s);
+        return launch_gemm_wreg<CMX_FMT_E4M3, kEpiStoreFp16, TM>(p, max_m_tiles, s);
     }
-    if (p.out_type == CMX_OUT_BF16) return launch_gemm_wreg<CMX_FMT_E5M2, kEpiStoreBf16>(p, max_m_tiles, s);
-    return launch_gemm_wreg<CMX_FMT_E5M2, kEpiStoreFp16>(p, max_m_tiles, s);
+    if (p.out_type == CMX_OUT_BF16) return launch_gemm_wreg<CMX_FMT_E5M2, kEpiStoreBf16, TM>(p, max_m_tiles, s);
+    return launch_gemm_wreg<CMX_FMT_E5M2, kEpiStoreFp16, TM>(p, max_m_tiles, s);
 }
 
 int check_operands(const void* a, uint32_t lda, const void* as, uint32_t ld_as, const void* w, uint32_t ldw,
@@ -1257,6 +1261,12 @@ bool scales_dword_aligned(const void* as, uint32_t ld_as, const void* ws, uint32
 #ifdef CMX_TEST_HOOKS
 extern "C" int cmx_debug_disable_streaming(int off) {
     cmx::g_disable_dl = off != 0;
+    return CMX_OK;
+}
+
+// pin the tile height (256 or 288 rows) of every later matmul call on pre-tiled weights (0 restores the heuristic)
+extern "C" int cmx_debug_pretiled_tile_rows(int rows) {
+    cmx::g_pretiled_tile_rows = rows == 256 || rows == 288 ? rows : 0;
     return CMX_OK;
 }
 
@@ -1314,7 +1324,9 @@ int gmm_common(GemmParams& p, const int32_t* group_sizes, uint32_t groups, uint3
         if (int rc = check_pretiled(p, fmt, swiglu); rc != CMX_OK) return rc;
     // average rows per group steers the tile height
     TileChoice t = choose_tile(ceil_div(m_total, groups), p.n, fmt, true);
-    if (p.w_pretiled) t = {256, 256, 5};     // the weights-to-registers kernel: 256 x 256 tiles, drawn from the counters
+    // the weights-to-registers kernel, tiles drawn from the counters: 256 x 288 when the groups average less than four
+    // tiles of rows (a group of 257 to 288 rows then takes one pass over its weights instead of two), else 256 x 256
+    if (p.w_pretiled) t = {256, g_pretiled_tile_rows ? g_pretiled_tile_rows : (ceil_div(m_total, groups) < 1024 ? 288 : 256), 5};
     int32_t* row_off = static_cast<int32_t*>(workspace);
     int32_t* tile_pref = row_off + (groups + 1);
     int32_t* tile_ctr = tile_pref + (groups + 1);
@@ -1330,7 +1342,7 @@ int gmm_common(GemmParams& p, const int32_t* group_sizes, uint32_t groups, uint3
     p.groups = groups;
     p.w_tiles = swiglu ? ceil_div(p.n / 2, t.tw / 2) : ceil_div(p.n, t.tw);
     const uint32_t max_m_tiles = m_total / t.tm + groups;
-    if (p.w_pretiled) return launch_pretiled(p, fmt, swiglu, max_m_tiles, s);
+    if (p.w_pretiled) return t.tm == 288 ? launch_pretiled<288>(p, fmt, swiglu, max_m_tiles, s) : launch_pretiled<256>(p, fmt, swiglu, max_m_tiles, s);
     if (swiglu && p.act_bf16 != nullptr) return dispatch_tile<CMX_FMT_E4M3, kEpiSwigluQuantAct>(p, t, max_m_tiles, s);
     if (swiglu) return dispatch_tile<CMX_FMT_E4M3, kEpiSwigluQuant>(p, t, max_m_tiles, s);
     switch (fmt) {

@@ -57,44 +57,56 @@ __device__ __forceinline__ void shift_scale(uint32_t& r, uint32_t sh) {
     asm volatile("v_lshrrev_b32 %0, %1, %0" : "+v"(r) : "v"(sh));
 }
 
-// acc += W-fragment x A-fragment with scale byte BYTE (0 or 2) of both scale registers; BIT as in mfma_acc
-#define CMX_WREG_MFMA(SELTXT, EXTRA)                                                                            \
-    if constexpr (BIT < 0)                                                                                      \
-        asm volatile("v_mfma_scale_f32_32x32x64_f8f6f4 %0, %1, %2, %0, %3, %4 " SELTXT EXTRA                    \
-                     : "+a"(acc) : "v"(w), "v"(a), "v"(sw), "v"(sa));                                           \
-    else                                                                                                        \
-        asm volatile("s_bitcmp1_b32 %5, %6\n\ts_cbranch_scc0 .Lskip%=\n\t"                                      \
-                     "v_mfma_scale_f32_32x32x64_f8f6f4 %0, %1, %2, %0, %3, %4 " SELTXT EXTRA                    \
-                     "\n.Lskip%=:"                                                                              \
-                     : "+a"(acc) : "v"(w), "v"(a), "v"(sw), "v"(sa), "s"(live), "n"(BIT < 0 ? 0 : BIT) : "scc")
+// acc += W-fragment x A-fragment with scale byte BYTE (0 or 2) of both scale registers; BIT as in mfma_acc.  The
+// accumulators of fragments 0..7 live in the 256 accumulation registers, which they fill; a ninth fragment's (BIT = 8, the
+// 288-row tile) in ordinary vector registers, which the MFMA takes as well.
+#define CMX_WREG_MFMA(ACC, SELTXT, EXTRA)                                                                       \
+    asm volatile("s_bitcmp1_b32 %5, %6\n\ts_cbranch_scc0 .Lskip%=\n\t"                                          \
+                 "v_mfma_scale_f32_32x32x64_f8f6f4 %0, %1, %2, %0, %3, %4 " SELTXT EXTRA                        \
+                 "\n.Lskip%=:"                                                                                  \
+                 : ACC(acc) : "v"(w), "v"(a), "v"(sw), "v"(sa), "s"(live), "n"(BIT) : "scc")
+#define CMX_WREG_MFMA_SEL(ACC, EXTRA)                                                                           \
+    if constexpr (BYTE == 0) { CMX_WREG_MFMA(ACC, "op_sel_hi:[0,0,0]", EXTRA); } else { CMX_WREG_MFMA(ACC, "op_sel_hi:[1,1,0]", EXTRA); }
 template <int FMT, int BYTE, int BIT>
 __device__ __forceinline__ void mfma_acc_b01(v16f& acc, const v8i& w, const v8i& a, uint32_t sw, uint32_t sa, uint32_t live) {
     static_assert(BYTE == 0 || BYTE == 2, "scale byte");
+    static_assert(BIT >= 0 && BIT < 32, "fragment");
     live = __builtin_amdgcn_readfirstlane(live);
     if constexpr (FMT == CMX_FMT_E4M3) {
-        if constexpr (BYTE == 0) { CMX_WREG_MFMA("op_sel_hi:[0,0,0]", ""); } else { CMX_WREG_MFMA("op_sel_hi:[1,1,0]", ""); }
+        if constexpr (BIT < 8) { CMX_WREG_MFMA_SEL("+a", ""); } else { CMX_WREG_MFMA_SEL("+v", ""); }
     } else {
-        if constexpr (BYTE == 0) { CMX_WREG_MFMA("op_sel_hi:[0,0,0]", " cbsz:1 blgp:1"); } else { CMX_WREG_MFMA("op_sel_hi:[1,1,0]", " cbsz:1 blgp:1"); }
+        if constexpr (BIT < 8) { CMX_WREG_MFMA_SEL("+a", " cbsz:1 blgp:1"); } else { CMX_WREG_MFMA_SEL("+v", " cbsz:1 blgp:1"); }
     }
 }
+#undef CMX_WREG_MFMA_SEL
 #undef CMX_WREG_MFMA
 
-// LDS footprint: activation ring (four slots of 256 rows), ring of two scale blocks (16 bytes per row of both operands),
-// next-tile mailbox
-constexpr size_t kWregLdsBytes = (size_t)4 * 256 * 128 + (size_t)2 * 512 * 16 + 512;
+// Tile heights.  256 rows: eight activation fragments per wavefront, all resident in registers (each refreshed in place), the
+// scales of both operands through the LDS.  288 rows: groups of up to 288 rows -- what a router that aims at 256 per expert
+// mostly produces -- take one tile where the first shape needs a second one that streams the whole weight panel again for a
+// few rows.  Nine fragments: their accumulators leave room for a window of three fragment buffers only (fragment j + 3 is
+// read when pair j has been issued), and the LDS (four slots of 36 KiB) for the activation scales only, so the weight
+// scales of a four-slab block are loaded straight into registers, 16 bytes per weight row and lane.
+__host__ __device__ constexpr bool wreg_wscale_regs(int tm) { return tm != 256; }
+__host__ __device__ constexpr int wreg_window(int tm) { return tm == 256 ? 8 : 3; }
+__host__ __device__ constexpr int wreg_scale_rows_padded(int tm) { return ((wreg_wscale_regs(tm) ? 0 : 256) + tm + 63) / 64 * 64; }
+// LDS footprint: activation ring (four slots), ring of two scale blocks (16 bytes per row), next-tile mailbox
+__host__ __device__ constexpr size_t wreg_lds_bytes(int tm) { return (size_t)4 * tm * 128 + (size_t)2 * wreg_scale_rows_padded(tm) * 16 + 512; }
 
 // LDS operations issued behind MFMA pair p of a step of kind K (0: first half of a slab, 1: second half): two fragment
-// reads; in the second half preceded by the scale read of that fragment for the next slab, and behind pair 0 by the two
-// weight scale reads as well.
-__host__ __device__ constexpr int wreg_lds_ops(int kind, int p) { return kind == 0 ? 2 : (3 + (p == 0 ? 2 : 0)); }
-// lgkmcnt that guarantees fragment j of a step of kind K (and with it the scale read before it) has landed, asked right
-// before pair j: LDS returns in order, so it is the number of operations issued after the reads of fragment j -- the rest
-// of the previous step (kind 1 - K) and pairs 0..j-1 of this one.  The counter has four bits: a smaller count only asks for
-// older reads as well.
-__host__ __device__ constexpr int wreg_frag_wait(int kind, int j, int fm) {
+// reads; in the second half preceded by the activation scale read of fragment p for the next slab, and behind pair 0 by the
+// two weight scale reads as well when those go through the LDS.
+__host__ __device__ constexpr int wreg_lds_ops(int kind, int p, bool wscale_regs) { return kind == 0 ? 2 : (3 + (p == 0 && !wscale_regs ? 2 : 0)); }
+// lgkmcnt that guarantees fragment j of a step of kind K has landed, asked right before pair j.  With a window of `win`
+// fragment buffers the reads of fragment j were the last operations behind the pair `win` pairs earlier (in this step or
+// the previous one); LDS returns in order, so the count is that of the operations behind the win - 1 pairs since.  (The
+// scale read of fragment j is older still.)  The counter has four bits: a smaller count only asks for older reads as well.
+__host__ __device__ constexpr int wreg_frag_wait(int kind, int j, int fm, int win, bool wscale_regs) {
     int n = 0;
-    for (int p = j + 1; p < fm; ++p) n += wreg_lds_ops(1 - kind, p);
-    for (int p = 0; p < j; ++p) n += wreg_lds_ops(kind, p);
+    for (int d = 1; d < win; ++d) {
+        const int q = j - d;
+        n += q >= 0 ? wreg_lds_ops(kind, q, wscale_regs) : wreg_lds_ops(1 - kind, q + fm, wscale_regs);
+    }
     return n < 15 ? n : 15;
 }
 // loads behind pair j when `total` loads are spread over `pairs` pairs: indices [first, first + count)
@@ -104,21 +116,26 @@ __host__ __device__ constexpr int wreg_first_load(int total, int pairs, int j) {
 // 256 x 128 bytes per slab and tile, so that a weight load of a wavefront reads 1 KiB of consecutive bytes (eight whole cache
 // lines); from row-major weights the same load takes 32 bytes from each of 32 rows, and that many more visits to the
 // vector cache made the kernel a quarter slower than the two-slot ones.
-template <int FMT, int EPI>
+template <int FMT, int EPI, int TM>
 __global__ __launch_bounds__(256) void mx_gemm_wreg_kernel(const GemmParams p) {
     static_assert(FMT == CMX_FMT_E4M3 || FMT == CMX_FMT_E5M2, "8-bit element formats only");
     static_assert(EPI != kEpiStore, "persistent kernel: SwiGLU or lean 16-bit store epilogue");
-    constexpr int TW = 256, TM = 256, NW = 4, WW = 4, WM = 1, FW = 2;
-    constexpr int NA = TM / 32;                                // activation fragments of the tile
-    constexpr int FM = (NA + WM - 1) / WM;                     // ... of a wavefront (fragment j of wavefront-row wm is fragment j * WM + wm of the tile)
+    static_assert(TM == 256 || TM == 288, "tile height");
+    constexpr int TW = 256, NW = 4, WW = 4, WM = 1, FW = 2;
+    constexpr int FM = TM / 32;                                // activation fragments of the tile = of every wavefront
+    constexpr int FMW = wreg_window(TM);                       // fragment buffers: fragment j lives in buffer j % FMW
+    constexpr bool kWScaleRegs = wreg_wscale_regs(TM);
+    static_assert(FM % FMW == 0 && FMW <= FM, "a fragment keeps its buffer from step to step");
     constexpr int kRing = 4;                                   // slabs in the weight register ring = slots of the activation ring
     constexpr int kSlotBytes = TM * kSlabBytes;
     constexpr int kScaleBase = kRing * kSlotBytes;
-    constexpr int kScaleRows = TW + TM;
+    constexpr int kScaleWRows = kWScaleRegs ? 0 : TW;          // weight rows in an LDS scale block
+    constexpr int kScaleRows = kScaleWRows + TM;
     constexpr int kALoads = TM / (8 * NW);                     // LDS-DMA loads per wavefront and slab
     constexpr int kWLoads = 8;                                 // weight loads per wavefront and slab: 2 steps x 2 fragments x 2 register halves
     constexpr int kSlabLoads = kALoads + kWLoads;
-    static_assert(WW * WM == NW && TW % (WW * 32) == 0 && TM % 32 == 0, "tile geometry");
+    constexpr int kBlockLoads = kWScaleRegs ? 2 + FW : 2;      // loads that go out with a scale block
+    static_assert(WW * WM == NW && TW % (WW * 32) == 0 && TM % (8 * NW) == 0, "tile geometry");
 
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t*)smem;
@@ -165,7 +182,8 @@ __global__ __launch_bounds__(256) void mx_gemm_wreg_kernel(const GemmParams p) {
 
     // descriptors of the tile whose slabs the load streams are requesting
     v4i w_rs, a_rs, s_rs[2];
-    uint32_t sgoff[2];
+    v4i ws_rs;                                  // weight scale rows of the tile's group (weight scales in registers)
+    uint32_t sgoff[2], wsgoff[FW];
     uint32_t a_last = 0;                        // last valid activation row of that tile
     auto wrow_of = [&](const Tile& t, uint32_t r) -> uint32_t {
         uint32_t gr;
@@ -185,20 +203,26 @@ __global__ __launch_bounds__(256) void mx_gemm_wreg_kernel(const GemmParams p) {
         t.mt = __builtin_amdgcn_readfirstlane(t.mt); t.row0 = __builtin_amdgcn_readfirstlane(t.row0);
         t.rows_valid = __builtin_amdgcn_readfirstlane(t.rows_valid);
     };
-    // Scale blocks: the rows of both operands form one sequence (weight rows, then activation rows) that is fetched in
-    // loads of 64 rows, two per wavefront: loads `wave` and `wave + 4` (where there is no such load, the first again).
+    // Scale blocks in the LDS: the rows of both operands form one sequence (weight rows, unless those go to registers, then
+    // activation rows) that is fetched in loads of 64 rows, two per wavefront: loads `wave` and `wave + 4` (where there is no
+    // such load, the first again).
     constexpr int kScaleLoads = (kScaleRows + 63) / 64;
     constexpr int kScaleRowsPadded = kScaleLoads * 64;
     constexpr int kScaleSlotBytesP = kScaleRowsPadded * 16;
     const uint32_t sload[2] = {wave, wave + 4 < (uint32_t)kScaleLoads ? wave + 4 : wave};
     auto aim_scales_at = [&](const Tile& t) {
-        const v4i ws_rs = make_rsrc(p.w_scale + (size_t)t.g * p.n * p.ld_ws);
+        ws_rs = make_rsrc(p.w_scale + (size_t)t.g * p.n * p.ld_ws);
         const v4i as_rs = make_rsrc(p.a_scale + (size_t)t.row0 * p.ld_as);
+        if constexpr (kWScaleRegs) {
+            // lane l of either half-wave: the scale row of the weight row it feeds to the MFMA as row l % 32 of fragment f
+#pragma unroll
+            for (int f = 0; f < FW; ++f) wsgoff[f] = mul_lo_u32(wrow_of(t, w_row_base + CMX_WREG_WOFF(f) + l32), p.ld_ws);
+        }
 #pragma unroll
         for (int k = 0; k < 2; ++k) {
             const uint32_t c = 64 * sload[k] + lane;
-            const bool is_w = 64 * sload[k] < (uint32_t)TW;              // uniform: TW is a multiple of 64
-            const uint32_t ar = c - TW < t.rows_valid ? c - TW : t.rows_valid - 1;
+            const bool is_w = 64 * sload[k] < (uint32_t)kScaleWRows;     // uniform: the weight rows are a multiple of 64
+            const uint32_t ar = c - kScaleWRows < t.rows_valid ? c - kScaleWRows : t.rows_valid - 1;
             sgoff[k] = is_w ? wrow_of(t, c) * p.ld_ws : ar * p.ld_as;
 #pragma unroll
             for (int q = 0; q < 4; ++q) s_rs[k][q] = is_w ? ws_rs[q] : as_rs[q];
@@ -257,29 +281,38 @@ __global__ __launch_bounds__(256) void mx_gemm_wreg_kernel(const GemmParams p) {
         dma_b128(dma_base + slot * kSlotBytes + i * (NW * 1024), off, a_rs, koff);
     };
     uint32_t blocks_issued = 0;                 // running count over all tiles: ring position = count & 1
+    v4i wsn[FW];                                // weight scales of the next four-slab block as they come from memory
+    uint32_t wsc[FW][4];                        // ... of the current block, one register per slab, shifted for this half-wave
     auto issue_scale_block = [&](uint32_t byte_off) {
         const uint32_t pos = blocks_issued & 1u;
         ++blocks_issued;
+        (void)wsn, (void)wsgoff;
         dma_b128(sdma_base[0] + pos * kScaleSlotBytesP, sgoff[0], s_rs[0], byte_off);
         dma_b128(sdma_base[1] + pos * kScaleSlotBytesP, sgoff[1], s_rs[1], byte_off);
+        if constexpr (kWScaleRegs) {
+#pragma unroll
+            for (int f = 0; f < FW; ++f) wsn[f] = wreg_load_b128<0>(wsgoff[f], ws_rs, byte_off);
+        }
     };
 
     // ---- fragment and scale read addresses -----------------------------------------------------------------------
     // a lane reads, for step h, the 16-byte chunks 4 h + lh (32-block 2h of the slab) and 4 h + 2 + lh (block 2h + 1) of its
-    // row.  One set of four base registers serves all slots: it points at the slot being read and is moved on between the
-    // two steps of a slab (the reads of step 1 already go to the next slab's slot); the immediate picks the fragment.
+    // row.  One set of four base registers serves all slots; the immediate picks the fragment.  The two bases of step 0 point
+    // at the slot of slab s while step 0 of slab s is multiplied and move on to the next slot between the two steps (the last
+    // reads behind the pairs of step 1 fetch the first fragments of slab s + 1); those of step 1 move on after step 1.
     const uint32_t x = (l32 & 7u) ^ ((l32 >> 3) & 1u);
     uint32_t ab[4];                             // [2 * step + half]
 #pragma unroll
     for (int j = 0; j < 4; ++j) ab[j] = lds0 + (wm * 32 + l32) * kSlabBytes + ((4 * (j >> 1) + 2 * (j & 1) + lh) ^ x) * 16;
-    auto move_read_base = [&](int delta) {
+    // the bases of step `step` move on to the next slot
+    auto move_read_base = [&](int step, int delta) {
         (void)ab;
 #pragma unroll
-        for (int j = 0; j < 4; ++j) asm volatile("v_add_u32 %0, %1, %0" : "+v"(ab[j]) : "s"(delta));
+        for (int j = 0; j < 2; ++j) asm volatile("v_add_u32 %0, %1, %0" : "+v"(ab[2 * step + j]) : "s"(delta));
     };
     // scale dword of the row (the lanes of half-wave lh use its bytes lh and lh + 2: see shift_scale)
     const uint32_t swb = lds0 + kScaleBase + (w_row_base + l32) * 16;
-    const uint32_t sab = lds0 + kScaleBase + (TW + wm * 32 + l32) * 16;
+    const uint32_t sab = lds0 + kScaleBase + (kScaleWRows + wm * 32 + l32) * 16;
     const uint32_t sshift = 8 * lh;
     uint32_t blocks_read = 0;                   // running count of the scale blocks whose first slab has been read
 
@@ -292,8 +325,8 @@ __global__ __launch_bounds__(256) void mx_gemm_wreg_kernel(const GemmParams p) {
             for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
 
     v4i wlo[kRing][2][FW], whi[kRing][2][FW];           // weight ring: [slab position][step][fragment], registers 0-3 / 4-7
-    v4i alo[FM], ahi[FM];                               // the activation fragments of the step being multiplied (refreshed in place)
-    uint32_t sw[2][FW];                                 // weight scales of a slab (bytes 0, 2: steps 0, 1), by slab parity
+    v4i alo[FMW], ahi[FMW];                             // activation fragment buffers: fragment j of a step in buffer j % FMW
+    uint32_t sw[2][FW];                                 // weight scales of a slab (bytes 0, 2: steps 0, 1), by slab parity (through the LDS)
     uint32_t sa[FM];                                    // activation scales, refreshed in place like the fragments
 
     using I0 = std::integral_constant<int, 0>;
@@ -307,12 +340,23 @@ __global__ __launch_bounds__(256) void mx_gemm_wreg_kernel(const GemmParams p) {
         v4i& dst = half ? whi[pos][h][f] : wlo[pos][h][f];
         dst = wreg_load_b128<(f * 2 + half) * 1024>(woff[h], w_rs, koff * TW);
     };
-    // one 16-byte read of this wavefront's activation fragment j for step `step` from the slot the base registers point at
+    // one 16-byte read of this wavefront's activation fragment j for step `step` from the slot the base registers of that step
+    // point at
     auto read_a_half = [&](auto step_c, auto j_c, auto half_c) {
         constexpr int step = decltype(step_c)::value, j = decltype(j_c)::value, half = decltype(half_c)::value;
         (void)ab, (void)alo, (void)ahi;
-        v4i& dst = half ? ahi[j] : alo[j];
+        v4i& dst = half ? ahi[j % FMW] : alo[j % FMW];
         dst = lds_read_b128<j * WM * 32 * kSlabBytes>(ab[2 * step + half]);
+    };
+    // the two reads that go out behind pair j of step `step`: fragment j + FMW of that step while there is one, else fragment
+    // j + FMW - FM of the step after it (whose base registers already point at its slot)
+    auto read_behind = [&](auto step_c, auto j_c) {
+        constexpr int step = decltype(step_c)::value, j = decltype(j_c)::value;
+        constexpr int g = j + FMW;
+        using StepT = std::integral_constant<int, (g < FM ? step : 1 - step)>;
+        using FragT = std::integral_constant<int, (g < FM ? g : g - FM)>;
+        read_a_half(StepT{}, FragT{}, I0{});
+        read_a_half(StepT{}, FragT{}, I1{});
     };
     auto read_w_scale_at = [&](uint32_t swb_at, auto set_c, auto f_c) {
         constexpr int set = decltype(set_c)::value, f = decltype(f_c)::value;
@@ -347,10 +391,10 @@ __global__ __launch_bounds__(256) void mx_gemm_wreg_kernel(const GemmParams p) {
         static_for<0, kWLoads>([&](auto ic) { issue_w_load(sc_, ic, s * kSlabBytes); });
     });
     asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(kWLoads + 2 * kSlabLoads) : "memory");      // scale block 0 and the activations of slab 0 are in
-    static_for<0, FM>([&](auto fc) { read_a_half(I0{}, fc, I0{}); read_a_half(I0{}, fc, I1{}); });
+    static_for<0, FMW>([&](auto fc) { read_a_half(I0{}, fc, I0{}); read_a_half(I0{}, fc, I1{}); });
     {
         const uint32_t off = scale_read_offset(0);
-        static_for<0, FW>([&](auto fc) { read_w_scale_at(swb + off, I0{}, fc); });
+        if constexpr (!kWScaleRegs) static_for<0, FW>([&](auto fc) { read_w_scale_at(swb + off, I0{}, fc); });
         static_for<0, FM>([&](auto fc) { read_a_scale_at(sab + off, fc); });
     }
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
@@ -359,7 +403,8 @@ __global__ __launch_bounds__(256) void mx_gemm_wreg_kernel(const GemmParams p) {
         static_for<0, FW * FM>([&](auto ic) {
             constexpr int i = decltype(ic)::value;
             (void)acc;
-            asm volatile("s_nop 15\n\ts_nop 15" : "+a"(acc[i / FM][i % FM]));
+            if constexpr (i % FM < 8) asm volatile("s_nop 15\n\ts_nop 15" : "+a"(acc[i / FM][i % FM]));
+            else asm volatile("s_nop 15\n\ts_nop 15" : "+v"(acc[i / FM][i % FM]));
         });
     };
     fence_accumulators();
@@ -373,10 +418,18 @@ __global__ __launch_bounds__(256) void mx_gemm_wreg_kernel(const GemmParams p) {
         constexpr int kSet = P % 2, kNextSet = (P + 1) % 2;
         using LoadPosT = std::integral_constant<int, kLoadSlot>;
         using NextSetT = std::integral_constant<int, kNextSet>;
-        (void)acc, (void)sw, (void)sa, (void)wlo, (void)whi, (void)alo, (void)ahi, (void)live, (void)sshift;
+        (void)acc, (void)sw, (void)sa, (void)wlo, (void)whi, (void)alo, (void)ahi, (void)live, (void)sshift, (void)wsn, (void)wsc;
         // own activation loads (and scale block) of slab s + 1 have landed: younger are the weights of slab s + 1 and all of
         // slab s + 2 (plus the scale block that went out with it when that was a position-0 slab)
-        asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(kWLoads + kSlabLoads + (P == 1 ? 2 : 0)) : "memory");
+        asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(kWLoads + kSlabLoads + (P == 1 ? kBlockLoads : 0)) : "memory");
+        if constexpr (kWScaleRegs && P == 0) {
+            // the weight scales of this turn's block arrived a turn ago: one register per slab, shifted for this half-wave
+            static_for<0, FW * 4>([&](auto ic) {
+                constexpr int f = decltype(ic)::value / 4, d = decltype(ic)::value % 4;
+                (void)wsc, (void)wsn, (void)sshift;
+                asm volatile("v_lshrrev_b32 %0, %1, %2" : "=v"(wsc[f][d]) : "v"(sshift), "v"(wsn[f][d]));
+            });
+        }
         // scales of the next slab: dword (P + 1) % 4 of its block; a new block starts with the slab at position 0
         if constexpr (P == 3) ++blocks_read;
         const uint32_t sc_off = scale_read_offset((P + 1) % 4);
@@ -384,39 +437,37 @@ __global__ __launch_bounds__(256) void mx_gemm_wreg_kernel(const GemmParams p) {
         // ---- step 0 ----
         static_for<0, FM>([&](auto jc) {
             constexpr int j = decltype(jc)::value;
-            asm volatile("s_waitcnt lgkmcnt(%0)" ::"n"(wreg_frag_wait(0, j, FM)) : "memory");
-            // the scales of this slab were read as whole dwords (behind the pairs of the previous step): first use here
-            if constexpr (j == 0) {
+            asm volatile("s_waitcnt lgkmcnt(%0)" ::"n"(wreg_frag_wait(0, j, FM, FMW, kWScaleRegs)) : "memory");
+            // the scales of this slab were read from the LDS as whole dwords (behind the pairs of the previous step): first use here
+            if constexpr (j == 0 && !kWScaleRegs) {
                 shift_scale(sw[kSet][0], sshift);
                 shift_scale(sw[kSet][1], sshift);
             }
             shift_scale(sa[j], sshift);
-            const v8i a = join8(alo[j], ahi[j]);
-            mfma_acc_b01<FMT, 0, j>(acc[0][j], join8(wlo[P][0][0], whi[P][0][0]), a, sw[kSet][0], sa[j], live);
-            mfma_acc_b01<FMT, 0, j>(acc[1][j], join8(wlo[P][0][1], whi[P][0][1]), a, sw[kSet][1], sa[j], live);
-            read_a_half(I1{}, jc, I0{});
-            read_a_half(I1{}, jc, I1{});
+            const v8i a = join8(alo[j % FMW], ahi[j % FMW]);
+            mfma_acc_b01<FMT, 0, j>(acc[0][j], join8(wlo[P][0][0], whi[P][0][0]), a, kWScaleRegs ? wsc[0][P] : sw[kSet][0], sa[j], live);
+            mfma_acc_b01<FMT, 0, j>(acc[1][j], join8(wlo[P][0][1], whi[P][0][1]), a, kWScaleRegs ? wsc[1][P] : sw[kSet][1], sa[j], live);
+            read_behind(I0{}, jc);
             if constexpr (P == 0 && j == 0) issue_scale_block(sblk);
             static_for<wreg_first_load(kALoads, FM, j), wreg_first_load(kALoads, FM, j + 1)>([&](auto ic) { issue_a_load(LoadPosT{}, ic, koff); });
         });
-        // the fragment reads of step 1 go to the next slab's slot
-        move_read_base(P == 3 ? -3 * kSlotBytes : kSlotBytes);
+        move_read_base(0, P == 3 ? -3 * kSlotBytes : kSlotBytes);
         // ---- step 1 ----
         static_for<0, FM>([&](auto jc) {
             constexpr int j = decltype(jc)::value;
-            asm volatile("s_waitcnt lgkmcnt(%0)" ::"n"(wreg_frag_wait(1, j, FM)) : "memory");
-            const v8i a = join8(alo[j], ahi[j]);
-            mfma_acc_b01<FMT, 2, j>(acc[0][j], join8(wlo[P][1][0], whi[P][1][0]), a, sw[kSet][0], sa[j], live);
-            mfma_acc_b01<FMT, 2, j>(acc[1][j], join8(wlo[P][1][1], whi[P][1][1]), a, sw[kSet][1], sa[j], live);
-            if constexpr (j == 0) {
+            asm volatile("s_waitcnt lgkmcnt(%0)" ::"n"(wreg_frag_wait(1, j, FM, FMW, kWScaleRegs)) : "memory");
+            const v8i a = join8(alo[j % FMW], ahi[j % FMW]);
+            mfma_acc_b01<FMT, 2, j>(acc[0][j], join8(wlo[P][1][0], whi[P][1][0]), a, kWScaleRegs ? wsc[0][P] : sw[kSet][0], sa[j], live);
+            mfma_acc_b01<FMT, 2, j>(acc[1][j], join8(wlo[P][1][1], whi[P][1][1]), a, kWScaleRegs ? wsc[1][P] : sw[kSet][1], sa[j], live);
+            if constexpr (j == 0 && !kWScaleRegs) {
                 read_w_scale_at(swb_at, NextSetT{}, I0{});
                 read_w_scale_at(swb_at, NextSetT{}, I1{});
             }
             read_a_scale_at(sab_at, jc);
-            read_a_half(I0{}, jc, I0{});
-            read_a_half(I0{}, jc, I1{});
+            read_behind(I1{}, jc);
             static_for<wreg_first_load(kWLoads, FM, j), wreg_first_load(kWLoads, FM, j + 1)>([&](auto ic) { issue_w_load(LoadPosT{}, ic, koff); });
         });
+        move_read_base(1, P == 3 ? -3 * kSlotBytes : kSlotBytes);
     };
 
     // ---- persistent loop: four slabs per turn, tiles change between turns ------------------------------------------
@@ -485,8 +536,8 @@ __global__ __launch_bounds__(256) void mx_gemm_wreg_kernel(const GemmParams p) {
                     for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
             fence_accumulators();
             // first fragments of the new tile again (slot 0 has landed and is visible, and the base registers point at it;
-            // the scales of its slab 0 are already in their registers)
-            static_for<0, FM>([&](auto fc) { read_a_half(I0{}, fc, I0{}); read_a_half(I0{}, fc, I1{}); });
+            // the activation scales of its slab 0 are already in their registers, the weight scales in theirs or on their way)
+            static_for<0, FMW>([&](auto fc) { read_a_half(I0{}, fc, I0{}); read_a_half(I0{}, fc, I1{}); });
             asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
         }
     }

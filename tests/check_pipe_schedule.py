@@ -40,14 +40,19 @@ FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-Xclang", "-target-featu
 # persistent 2 x 2 kernels send all 8 weight loads early -- plus 2 prefetch loads in the persistent 2 x 2 kernels)
 #   mx_gemm_pipe_kernel<FMT, EPI, TM, WW, WM, NSLOT>; EPI 0 store, 1 SwiGLU + requant, 2 lean bf16, 4 lean fp16, 5 = 1 + bf16 activations
 #   mx_gemm_pipe_fp4_kernel<EPI, WW, WM>
-#   mx_gemm_wreg_kernel<FMT, EPI>: the wait at the start of a slab leaves the weight loads of the next slab and all loads of the
-#   one after in flight (8 + 16), two more behind the slab that sent a scale block
+#   mx_gemm_wreg_kernel<FMT, EPI, TM>: the wait at the start of a slab leaves the weight loads of the next slab and all loads of
+#   the one after in flight (8 + 16 or 17), and behind the slab that sent a scale block the loads of that block too
 KERNELS = [
-    ("mx_gemm_wreg_kernel<0, 1>", {24, 26}),
-    ("mx_gemm_wreg_kernel<0, 2>", {24, 26}),
-    ("mx_gemm_wreg_kernel<0, 4>", {24, 26}),
-    ("mx_gemm_wreg_kernel<1, 2>", {24, 26}),
-    ("mx_gemm_wreg_kernel<1, 4>", {24, 26}),
+    ("mx_gemm_wreg_kernel<0, 1, 256>", {24, 26}),
+    ("mx_gemm_wreg_kernel<0, 2, 256>", {24, 26}),
+    ("mx_gemm_wreg_kernel<0, 4, 256>", {24, 26}),
+    ("mx_gemm_wreg_kernel<1, 2, 256>", {24, 26}),
+    ("mx_gemm_wreg_kernel<1, 4, 256>", {24, 26}),
+    ("mx_gemm_wreg_kernel<0, 1, 288>", {25, 29}),               # nine activation loads per slab; four loads go out with a scale block
+    ("mx_gemm_wreg_kernel<0, 2, 288>", {25, 29}),
+    ("mx_gemm_wreg_kernel<0, 4, 288>", {25, 29}),
+    ("mx_gemm_wreg_kernel<1, 2, 288>", {25, 29}),
+    ("mx_gemm_wreg_kernel<1, 4, 288>", {25, 29}),
     ("mx_gemm_pipe_kernel<0, 1, 256, 2, 2, 2>", {10}),
     ("mx_gemm_pipe_kernel<0, 1, 256, 4, 1, 2>", {8}),
     ("mx_gemm_pipe_kernel<0, 5, 256, 2, 2, 2>", {10}),          # SwiGLU + requant that also writes the bf16 activations

@@ -43,6 +43,7 @@ _HOOKS = {
     "cmx_mfma_raw_probe": (_C.c_int, [_C.c_void_p] * 5 + [_C.c_int] * 3 + [_C.c_void_p]),
     "cmx_debug_force_tile": (_C.c_int, [_C.c_int] * 3),
     "cmx_debug_disable_streaming": (_C.c_int, [_C.c_int]),
+    "cmx_debug_pretiled_tile_rows": (_C.c_int, [_C.c_int]),
 }
 _test_lib = None
 
@@ -71,6 +72,7 @@ class hooked_library:
         from catccos_amd import _lib
         self.lib.cmx_debug_force_tile(0, 0, 0)
         self.lib.cmx_debug_disable_streaming(0)
+        self.lib.cmx_debug_pretiled_tile_rows(0)
         _lib.activate(self.prev)
         return False
 

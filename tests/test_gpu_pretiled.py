@@ -7,9 +7,25 @@ import torch
 
 from oracle import mx_oracle as O
 from catccos_amd import workloads as W
-from tests.gpu_util import dev, host, bf16_dev, close_bf16
+from tests.gpu_util import dev, host, bf16_dev, close_bf16, hooked_library, hooks_lib
 
 pytestmark = pytest.mark.gpu
+
+# tile heights of the kernel behind the pre-tiled entry points: None leaves the choice to the product library (288 rows
+# for groups that average less than 1024 rows, else 256); the others pin it on the test build of the library
+TILE_HEIGHTS = [None, 256, 288]
+
+
+@pytest.fixture(autouse=True)
+def _tile_height(request):
+    params = getattr(getattr(request.node, "callspec", None), "params", {})
+    tm = params.get("tm")
+    if tm is None:
+        yield
+        return
+    with hooked_library():
+        hooks_lib().cmx_debug_pretiled_tile_rows(tm)
+        yield
 
 
 def pretile_numpy(w: np.ndarray, pair_gate_up: bool) -> np.ndarray:
@@ -57,9 +73,10 @@ def _weights(rng, g, n, k, std, fmt="E4M3"):
     return np.stack([q for q, _ in qs]), np.stack([s for _, s in qs])
 
 
+@pytest.mark.parametrize("tm", TILE_HEIGHTS)
 @pytest.mark.parametrize("fmt,out", [("E4M3", "bf16"), ("E5M2", "fp16")])
-@pytest.mark.parametrize("counts", [[5, 0, 300, 1, 0, 257, 64], [0, 0, 7], [512], [1] * 9])
-def test_gmm_on_pretiled_weights(fmt, out, counts):
+@pytest.mark.parametrize("counts", [[5, 0, 300, 1, 0, 257, 64], [0, 0, 7], [512], [1] * 9, [288, 289, 287, 0, 576]])
+def test_gmm_on_pretiled_weights(tm, fmt, out, counts):
     from catccos_amd import ops
     rng = np.random.default_rng(sum(counts) + 1)
     n, k = 320, 512
@@ -83,7 +100,8 @@ def test_gmm_on_pretiled_weights(fmt, out, counts):
     assert torch.equal(c.view(torch.int16), c_rm.view(torch.int16))
 
 
-def test_gmm1_and_gmm2_on_pretiled_weights_many_ragged_groups():
+@pytest.mark.parametrize("tm", TILE_HEIGHTS)
+def test_gmm1_and_gmm2_on_pretiled_weights_many_ragged_groups(tm):
     """43 groups (empty, whole-tile, ragged) at one weight tile per group: fewer tiles than workgroups, so every tile is
     cut into row parts that different workgroups compute; every row must still come out once, with the bits of the
     row-major kernels, and agree with the oracle."""
@@ -114,8 +132,9 @@ def test_gmm1_and_gmm2_on_pretiled_weights_many_ragged_groups():
     assert torch.equal(codes, codes_r) and torch.equal(scales, scales_r)
 
 
+@pytest.mark.parametrize("tm", TILE_HEIGHTS)
 @pytest.mark.parametrize("groups,n", [(60, 1280), (70, 1024)])
-def test_pretiled_more_tiles_than_workgroups(groups, n):
+def test_pretiled_more_tiles_than_workgroups(tm, groups, n):
     """Several rounds of tiles per workgroup (tiles drawn from the per-XCD counters while the load streams of the
     previous tile are still running) and a partly filled last round, bit for bit against the row-major kernels on
     GPU-made operands; sampled rows against the oracle."""
@@ -173,8 +192,9 @@ def _ffn_inputs(tokens, k, n, experts, top_k, seed):
     return x, idx, p, w1q, w1s, w2q, w2s
 
 
+@pytest.mark.parametrize("tm", TILE_HEIGHTS)
 @pytest.mark.parametrize("tokens,k,n,experts,top_k", [(64, 512, 1024, 16, 6), (777, 512, 2048, 8, 8)])
-def test_ffn_on_pretiled_weights(tokens, k, n, experts, top_k):
+def test_ffn_on_pretiled_weights(tm, tokens, k, n, experts, top_k):
     from catccos_amd import ops
     x, idx, p, w1q, w1s, w2q, w2s = _ffn_inputs(tokens, k, n, experts, top_k, tokens)
     w1, w2 = dev(w1q), dev(w2q)
@@ -198,3 +218,22 @@ def test_pretiled_ffn_rejects_bad_shapes():
     args = [t.data_ptr() for t in (bf16_dev(x), dev(idx), dev(p), dev(w1q), dev(w1s), dev(w2q), dev(w2s), out, ws)]
     assert lib.cmx_dispatch_ffn_combine_pretiled(None, *args, 8, 512, 512, 4, 2) == -1
     assert b"N % 1024" in lib.cmx_last_error()
+
+
+def test_pretiled_long_groups_take_the_256_row_tile():
+    """Groups that average 1024 rows or more: the product library picks the 256-row tile (several tiles per group and
+    weight panel, the last one ragged); bit for bit against the row-major kernels."""
+    from catccos_amd import ops
+    k, n, groups = 512, 512, 3
+    g = torch.Generator(device="cuda")
+    g.manual_seed(11)
+    counts_h = np.array([1500, 700, 1100], dtype=np.int32)
+    m = int(counts_h.sum())
+    a, a_s = ops.mx_quant(torch.randn((m, k), generator=g, device="cuda").to(torch.bfloat16), "E4M3", "rne")
+    w, w_s = ops.mx_quant((torch.randn((groups * n, k), generator=g, device="cuda") * 0.05).to(torch.bfloat16), "E4M3", "lut")
+    w, w_s = w.view(groups, n, k), w_s.view(groups, n, -1)
+    cnt = torch.from_numpy(counts_h).cuda()
+    assert torch.equal(ops.mx_gmm(a, a_s, ops.pretile_weights(w, False), w_s, cnt, k), ops.mx_gmm(a, a_s, w, w_s, cnt, k))
+    c1, s1, _ = ops.mx_gmm_swiglu_quant(a, a_s, ops.pretile_weights(w, True), w_s, cnt, k)
+    c2, s2, _ = ops.mx_gmm_swiglu_quant(a, a_s, w, w_s, cnt, k)
+    assert torch.equal(c1, c2) and torch.equal(s1, s2)
