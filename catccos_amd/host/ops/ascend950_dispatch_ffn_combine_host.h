@@ -9,6 +9,21 @@
 
 class Ascend950DispatchFFNCombineOperator : public CatccosOperator {
 public:
+    // AllocateDeviceSpace is where this operator loads its weights, so it is also where they are brought into the order
+    // the fastest grouped kernels read (cmx_mx_pretile_weights, one pass): for the shapes that path covers, ptrB and the
+    // W2 pointer then hold tiled weights and Launch calls the pre-tiled entry point, whose output has the same bits.
+    static bool WeightsPretiled(const CocTilingParams& t) { return t.k % 512 == 0 && t.n % 1024 == 0; }
+
+    static uint8_t* Pretile(uint8_t* w, uint32_t experts, uint32_t rows, uint32_t cols, int pairGateUp)
+    {
+        const size_t bytes = cmx_mx_pretiled_weight_bytes(experts, rows, cols, pairGateUp);
+        uint8_t* tiled = mxrt::DeviceAlloc(bytes);
+        MX_CHECK(cmx_mx_pretile_weights(w, tiled, experts, rows, cols, pairGateUp, nullptr));
+        MX_CHECK(cmx_rt_stream_sync(nullptr));
+        MX_CHECK(cmx_rt_free(w));
+        return tiled;
+    }
+
     // Buffer order after AllocateDeviceSpace:
     //   ptrA = x bf16 [m,k], ptrB = W1 [E,n,k], ptrC = out bf16 [m,k],
     //   custom = { W2 [E,k,n/2], expertIdx i32 [m,topK], probs f32 [m,topK], W1 scale [E,n,k/32], W2 scale [E,k,n/64] }
@@ -40,6 +55,10 @@ public:
         uint8_t* probs = mxops::DeviceBufferFromFile(routeBytes, file("in_gather_gate_weight"));
         uint8_t* out = mxrt::DeviceAlloc(xBytes);
         MX_CHECK(cmx_rt_memset(out, 0, xBytes));
+        if (WeightsPretiled(t)) {
+            w1 = Pretile(w1, static_cast<uint32_t>(experts), t.n, t.k, 1);
+            w2 = Pretile(w2, static_cast<uint32_t>(experts), static_cast<uint32_t>(n2), static_cast<uint32_t>(k2), 0);
+        }
         params.SetKernelParams(x, w1, out, w2, expertIdx, probs, w1Scale, w2Scale);
     }
 
@@ -111,6 +130,14 @@ public:
     static int Launch(void* stream, const KernelParams& p, uint8_t* out, uint8_t* workspace, uint8_t* symmetric,
                       const CocTilingParams& t)
     {
+        if (WeightsPretiled(t)) {
+            if (t.rankSize != 1) {
+                return CMX_EINVAL;
+            }
+            return cmx_dispatch_ffn_combine_pretiled(stream, p.ptrA, p.customPtrs[1], p.customPtrs[2], p.ptrB, p.customPtrs[3],
+                                                     p.customPtrs[0], p.customPtrs[4], out, workspace, t.m, t.k, t.n,
+                                                     t.expertNum / t.epSize, t.topK);
+        }
         return catccos_ascend950_dispatch_ffn_combine(0, stream, 0, p.ptrA, p.customPtrs[1], p.customPtrs[2], p.ptrB,
                                                       p.customPtrs[3], p.customPtrs[0], p.customPtrs[4], out, workspace, symmetric,
                                                       t.m, t.k, t.n, t.expertNum / t.epSize, t.topK, static_cast<int>(t.rankSize));

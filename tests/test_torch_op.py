@@ -59,3 +59,33 @@ def test_ffn_op_matches_oracle_and_checks_arguments():
             torch.ops.catccos.ascend950_dispatch_ffn_combine(*bad)
     finally:
         assert torch.ops.catccos.finalize() == 0
+
+
+@pytest.mark.gpu
+def test_pretiled_ops_give_the_bits_of_the_reference_op():
+    import catccos_amd.torch_op  # noqa: F401
+    tokens, k, n, experts, top_k = 200, 512, 1024, 8, 4
+    rng = np.random.default_rng(19)
+    x = W.normal_bf16((tokens, k), 19)
+    idx, p = W.softmax_topk_routing(tokens, experts, top_k, 20)
+    w1 = [O.mx_quant(O.bf16_round(rng.standard_normal((n, k)).astype(np.float32) / np.sqrt(k)), "E4M3", "lut") for _ in range(experts)]
+    w2 = [O.mx_quant(O.bf16_round(rng.standard_normal((k, n // 2)).astype(np.float32) / np.sqrt(n // 2)), "E4M3", "lut") for _ in range(experts)]
+    dev = lambda a, dt: torch.from_numpy(np.ascontiguousarray(a)).cuda().view(dt)
+    args = [dev(x.view(np.int16), torch.bfloat16), dev(idx.astype(np.int32), torch.int32), dev(p.astype(np.float32), torch.float32),
+            dev(np.stack([a for a, _ in w1]), torch.float8_e4m3fn), dev(np.stack([b for _, b in w1]), torch.float8_e8m0fnu),
+            dev(np.stack([a for a, _ in w2]), torch.float8_e4m3fn), dev(np.stack([b for _, b in w2]), torch.float8_e8m0fnu)]
+    assert torch.ops.catccos.init(0, 1, 1 << 30, "tcp://127.0.0.1:1") == 0
+    try:
+        y = torch.ops.catccos.ascend950_dispatch_ffn_combine(*args)
+        w1t, w2t = torch.ops.catccos.ascend950_pretile_ffn_weights(args[3], args[5])
+        assert w1t.dtype == torch.uint8 and w1t.numel() == args[3].numel() and w2t.numel() == args[5].numel()
+        yt = torch.ops.catccos.ascend950_dispatch_ffn_combine_pretiled(args[0], args[1], args[2], w1t, args[4], w2t, args[6])
+        assert torch.equal(y, yt)
+        with pytest.raises(RuntimeError, match="wrong size"):
+            torch.ops.catccos.ascend950_dispatch_ffn_combine_pretiled(args[0], args[1], args[2], w1t[:-16], args[4], w2t, args[6])
+        with pytest.raises(RuntimeError, match="must have dtype"):
+            torch.ops.catccos.ascend950_dispatch_ffn_combine_pretiled(*args)       # row-major weights handed to the pre-tiled op
+        with pytest.raises(RuntimeError, match="divisible by 512"):
+            torch.ops.catccos.ascend950_pretile_ffn_weights(args[3][:, :, :256].contiguous(), args[5][:, :256].contiguous())
+    finally:
+        torch.ops.catccos.finalize()
