@@ -1,5 +1,6 @@
-// Hand-scheduled 256 x 256 block-scaled matmul kernel for the 8-bit MX formats whose weight fragments never pass
-// through the LDS (included by mx_gemm.hip after mx_gemm_pipe.h, whose helpers it shares).
+// Hand-scheduled grouped block-scaled matmul kernel for the 8-bit MX formats whose weight fragments never pass through the
+// LDS (included by mx_gemm.hip after mx_gemm_pipe.h, whose helpers it shares).  Tiles of 256 weight rows x 256 or 288
+// activation rows; what follows describes the 256-row form, "Tile heights" below what the taller one changes.
 //
 // For grouped problems with about one tile of rows per group every tile streams a weight panel of its own from HBM,
 // and what bounds the two-slot kernels there is how many weight bytes a CU can keep in flight: the LDS holds two
@@ -29,14 +30,14 @@
 //   step 1:  8 pairs; behind pair j the scale read and the two reads of fragment j of slab s + 1 (pair 0: also the two
 //            weight scales) and weight load j of slab s + 3
 // The K positions are multiplied and summed in the order of the two-slot kernels (step h of a slab takes its 32-blocks
-// 2h and 2h + 1), so the results are the same bits.  The lanes of half-wave
-// lh, whose scale byte applies to the first (lh = 0) or second (lh = 1) block of an MFMA, need bytes lh (step 0) and
-// 2 + lh (step 1) of the slab's dword: the dword is read whole, shifted right by one byte in the upper half-wave right
-// before its first use (one VALU instruction), and the MFMAs select bytes 0 and 2.  The activation scale of fragment j
-// is refreshed in place like the fragment itself.  (Measured alternatives at 256 groups of ~256 rows, K = 7168: reading
-// the dword at byte address lh, which the LDS allows, +5 % kernel time over no shift at all; the shift under a half EXEC
-// mask +4 %; this shift +2.5 %; pairing the blocks (h, 2 + h), which needs no shift but sums K in another order than the
-// other kernels and so differs from them in the last bit of one output in a million, +0.)
+// 2h and 2h + 1), so the results are the same bits.  The lanes of half-wave lh, whose scale byte applies to the first
+// (lh = 0) or second (lh = 1) block of an MFMA, need bytes lh (step 0) and 2 + lh (step 1) of the slab's dword: the dword
+// is read whole, shifted right by one byte in the upper half-wave right before its first use (one VALU instruction), and
+// the MFMAs select bytes 0 and 2.  The activation scale of fragment j is refreshed in place like the fragment itself.
+// (Measured alternatives at 256 groups of ~256 rows, K = 7168: reading the dword at byte address lh, which the LDS
+// allows, +5 % kernel time over no shift at all; the shift under a half EXEC mask +4 %; this shift +2.5 %; pairing the
+// blocks (h, 2 + h), which needs no shift but sums K in another order than the other kernels and so differs from them in
+// the last bit of one output in a million, +0.)
 // The kernel is persistent like the two-slot grouped kernels: one workgroup per CU draws tiles from its XCD's counter,
 // and the load streams run on into the next tile while the last slabs of a tile are multiplied.
 #pragma once
