@@ -63,3 +63,8 @@ def test_workspace_sizes_are_host_arithmetic():
     assert lib.cmx_mx_gmm_ex_workspace_bytes(16, 256, 512, 1) >= meta
     assert lib.cmx_mx_gmm_ex_workspace_bytes(16, 256, 512, 0) >= meta + 16 * 256 * (512 + 16)
     assert lib.cmx_int8_gmm_workspace_bytes(4, 256, 512, 0) >= lib.cmx_int8_gmm_workspace_bytes(4, 256, 512, 1) + 4 * 256 * 512
+    # pre-tiled weights: whole 256-row tiles (gate|up weights: 128 + 128 rows), 0 for shapes the layout does not cover
+    assert lib.cmx_mx_pretiled_weight_bytes(256, 4096, 7168, 1) == 256 * 4096 * 7168
+    assert lib.cmx_mx_pretiled_weight_bytes(3, 320, 512, 0) == 3 * 512 * 512
+    assert lib.cmx_mx_pretiled_weight_bytes(2, 640, 1024, 1) == 2 * 3 * 256 * 1024
+    assert lib.cmx_mx_pretiled_weight_bytes(2, 640, 256, 0) == 0 and lib.cmx_mx_pretiled_weight_bytes(2, 96, 512, 1) == 0
