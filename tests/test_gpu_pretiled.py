@@ -237,3 +237,33 @@ def test_pretiled_long_groups_take_the_256_row_tile():
     c1, s1, _ = ops.mx_gmm_swiglu_quant(a, a_s, ops.pretile_weights(w, True), w_s, cnt, k)
     c2, s2, _ = ops.mx_gmm_swiglu_quant(a, a_s, w, w_s, cnt, k)
     assert torch.equal(c1, c2) and torch.equal(s1, s2)
+
+
+@pytest.mark.parametrize("tm", TILE_HEIGHTS)
+def test_pretiled_gmm_with_row_pitches(tm):
+    """Activation, activation-scale and output rows at pitches larger than a row (what a caller's sub-view has): the bytes
+    between the rows are neither read into the result nor written."""
+    from catccos_amd import ops
+    rng = np.random.default_rng(21)
+    counts = [130, 0, 290, 33]
+    n, k = 512, 1024
+    m = sum(counts)
+    aq, asc = O.mx_quant(O.bf16_round(rng.standard_normal((m, k)).astype(np.float32)))
+    wq, ws = _weights(rng, len(counts), n, k, 1.0)
+    a_big = torch.full((m, k + 64), 0x7F, dtype=torch.uint8, device="cuda")            # 0x7F: NaN codes in the padding
+    a_big[:, :k] = dev(aq)
+    s_big = torch.full((m, k // 32 + 16), 0xFF, dtype=torch.uint8, device="cuda")      # 0xFF: NaN scales in the padding
+    s_big[:, :k // 32] = dev(asc)
+    c_big = torch.full((m, n + 24), 7.0, dtype=torch.bfloat16, device="cuda")
+    cnt = dev(np.array(counts, dtype=np.int32))
+    ops.mx_gmm(a_big[:, :k], s_big[:, :k // 32], ops.pretile_weights(dev(wq), False), dev(ws), cnt, k, c=c_big[:, :n])
+    bad, worst = close_bf16(host(c_big[:, :n].contiguous()), O.mx_gmm_f32(aq, asc, wq, ws, counts))
+    assert bad == 0, (bad, worst)
+    assert bool((c_big[:, n:].float() == 7.0).all())
+    codes = torch.full((m, n // 2 + 32), 0xEE, dtype=torch.uint8, device="cuda")
+    scales = torch.full((m, n // 64 + 6), 0xEE, dtype=torch.uint8, device="cuda")
+    ops.mx_gmm_swiglu_quant(a_big[:, :k], s_big[:, :k // 32], ops.pretile_weights(dev(wq), True), dev(ws), cnt, k,
+                            outs=(codes[:, :n // 2], scales[:, :n // 64]))
+    c_r, s_r, _ = ops.mx_gmm_swiglu_quant(dev(aq), dev(asc), dev(wq), dev(ws), cnt, k)
+    assert torch.equal(codes[:, :n // 2], c_r) and torch.equal(scales[:, :n // 64], s_r)
+    assert bool((codes[:, n // 2:] == 0xEE).all()) and bool((scales[:, n // 64:] == 0xEE).all())
