@@ -267,3 +267,34 @@ def test_pretiled_gmm_with_row_pitches(tm):
     c_r, s_r, _ = ops.mx_gmm_swiglu_quant(dev(aq), dev(asc), dev(wq), dev(ws), cnt, k)
     assert torch.equal(codes[:, :n // 2], c_r) and torch.equal(scales[:, :n // 64], s_r)
     assert bool((codes[:, n // 2:] == 0xEE).all()) and bool((scales[:, n // 64:] == 0xEE).all())
+
+
+@pytest.mark.parametrize("tm", [256, 288])
+def test_pretiled_seeded_sweep_matches_row_major_bits(tm):
+    """Thirty seeded problems (group counts 1..40, group sizes from empty to several tiles, N ragged against the 256-row
+    weight tile, K from one to six 512-byte blocks): both grouped matmuls on pre-tiled weights give the bits of the
+    row-major entry points, whose parity with the oracle the other suites establish."""
+    from catccos_amd import ops
+    rng = np.random.default_rng(1000 + tm)
+    g = torch.Generator(device="cuda")
+    for case in range(30):
+        groups = int(rng.integers(1, 41))
+        kind = case % 3
+        hi = (40, 300, 900)[kind]
+        counts_h = rng.integers(0, hi + 1, size=groups).astype(np.int32)
+        if counts_h.sum() == 0:
+            counts_h[0] = 17
+        m = int(counts_h.sum())
+        k = 512 * int(rng.integers(1, 7))
+        n = 64 * int(rng.integers(1, 21))
+        g.manual_seed(case)
+        a, a_s = ops.mx_quant(torch.randn((m, k), generator=g, device="cuda").to(torch.bfloat16), "E4M3", "rne")
+        w, w_s = ops.mx_quant((torch.randn((groups * n, k), generator=g, device="cuda") * 0.06).to(torch.bfloat16), "E4M3", "lut")
+        w, w_s = w.view(groups, n, k), w_s.view(groups, n, -1)
+        cnt = torch.from_numpy(counts_h).cuda()
+        what = (case, groups, m, n, k)
+        y_t = ops.mx_gmm(a, a_s, ops.pretile_weights(w, False), w_s, cnt, k)
+        assert torch.equal(y_t, ops.mx_gmm(a, a_s, w, w_s, cnt, k)), what
+        c_t, s_t, _ = ops.mx_gmm_swiglu_quant(a, a_s, ops.pretile_weights(w, True), w_s, cnt, k)
+        c_r, s_r, _ = ops.mx_gmm_swiglu_quant(a, a_s, w, w_s, cnt, k)
+        assert torch.equal(c_t, c_r) and torch.equal(s_t, s_r), what
