@@ -42,6 +42,15 @@ def test_host_only_entry_points_work_without_a_gpu():
     # a bad argument is reported through the error string, not a crash
     rc = lib.cmx_mx_quant(None, 0, None, 0, None, 0, 1, 33, 0, 0, None)
     assert rc != 0 and lib.cmx_last_error()
+    # the pre-tiled family validates on the host before anything is launched
+    assert lib.cmx_mx_pretile_weights(None, None, 2, 256, 512, 0, None) == -1 and b"null pointer" in lib.cmx_last_error()
+    assert lib.cmx_mx_pretile_weights(16, 32, 2, 256, 256, 0, None) == -1 and b"multiple of 512" in lib.cmx_last_error()
+    assert lib.cmx_mx_pretile_weights(16, 32, 2, 96, 512, 1, None) == -1 and b"multiple of 64" in lib.cmx_last_error()
+    assert lib.cmx_mx_pretile_weights(8, 32, 2, 256, 512, 0, None) == -1 and b"16-byte aligned" in lib.cmx_last_error()
+    assert lib.cmx_mx_pretile_weights(None, None, 0, 256, 512, 0, None) == 0           # nothing to do
+    assert lib.cmx_dispatch_ffn_combine_pretiled(None, 16, 16, 16, 16, 16, 16, 16, 16, 256, 8, 512, 512, 4, 2) == -1
+    assert b"N % 1024" in lib.cmx_last_error()
+    assert lib.cmx_dispatch_ffn_combine_pretiled(None, 16, 16, 16, 16, 16, 16, 16, 16, 256, 8, 768, 1024, 4, 2) == -1
 
 
 def test_header_is_plain_c(tmp_path):
