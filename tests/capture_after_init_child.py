@@ -1,6 +1,7 @@
 """Child process of test_gpu_ffn.test_capture_right_after_init: in a process that has launched none of the library's
-kernels, cmx_init() alone must be enough to capture the FFN chain and the allocation-free grouped matmul into a HIP
-graph (no kernel's first launch may need set-up that a capture forbids).  The graph is replayed twice, with eager
+kernels, cmx_init() alone must be enough to capture the FFN chain (on row-major and on pre-tiled weights) and the
+allocation-free grouped matmul into a HIP graph (no kernel's first launch may need set-up that a capture forbids; the
+one-off weight tiling pass runs before the capture, as it would at weight-load time).  The graph is replayed twice, with eager
 work in between, and every replay compared bit for bit with eager runs made afterwards.  Prints CAPTURE-OK."""
 import os
 import sys
@@ -18,7 +19,7 @@ from tests.gpu_util import dev, bf16_dev        # noqa: E402
 
 
 def main() -> int:
-    tokens, k, n, experts, top_k = 96, 512, 512, 8, 4
+    tokens, k, n, experts, top_k = 96, 512, 1024, 8, 4
     rng = np.random.default_rng(5)
     x = W.normal_bf16((tokens, k), 5)
     idx, p = W.softmax_topk_routing(tokens, experts, top_k, 6)
@@ -35,6 +36,8 @@ def main() -> int:
     ws = torch.empty(ops.ffn_workspace_bytes(tokens, k, n, experts, top_k), dtype=torch.uint8, device="cuda")
     ws_eager = torch.empty_like(ws)
     out = torch.zeros((tokens, k), dtype=torch.bfloat16, device="cuda")
+    out_t = torch.zeros((tokens, k), dtype=torch.bfloat16, device="cuda")
+    ws_t = torch.empty_like(ws)
     codes = torch.zeros((m, n // 2), dtype=torch.uint8, device="cuda")
     scales = torch.zeros((m, ops.scale_cols(n // 2)), dtype=torch.uint8, device="cuda")
 
@@ -42,7 +45,8 @@ def main() -> int:
         ops.dispatch_ffn_combine(xd, idxd, pd, w1d, w1sd, w2d, w2sd, workspace=w, out=o)
         ops.mx_gmm_swiglu_quant_noalloc(aqd, ascd, w1d, w1sd, cnt, k, c, s, None)
 
-    ops.init()                                   # the only library call before the capture
+    ops.init()                                   # the only library call before the capture, apart from the tiling pass
+    w1t, w2t = ops.pretile_weights(w1d, True), ops.pretile_weights(w2d, False)
     torch.cuda.synchronize()
     graph = torch.cuda.CUDAGraph()
     side = torch.cuda.Stream()
@@ -50,10 +54,12 @@ def main() -> int:
     with torch.cuda.stream(side):
         with torch.cuda.graph(graph, stream=side):
             run(out, ws, codes, scales)
+            ops.dispatch_ffn_combine(xd, idxd, pd, w1t, w1sd, w2t, w2sd, workspace=ws_t, out=out_t)
     torch.cuda.current_stream().wait_stream(side)
     for rep in range(2):
         xd.copy_(bf16_dev(W.normal_bf16((tokens, k), 200 + rep)))
         out.fill_(7.0)
+        out_t.fill_(7.0)
         codes.fill_(0xEE)
         scales.fill_(0xEE)
         graph.replay()
@@ -61,7 +67,8 @@ def main() -> int:
         e_out, e_codes, e_scales = torch.zeros_like(out), torch.zeros_like(codes), torch.zeros_like(scales)
         run(e_out, ws_eager, e_codes, e_scales)          # eager, after the replay (and between the replays)
         torch.cuda.synchronize()
-        if not (torch.equal(out.view(torch.int16), e_out.view(torch.int16)) and torch.equal(codes, e_codes) and torch.equal(scales, e_scales)):
+        if not (torch.equal(out.view(torch.int16), e_out.view(torch.int16)) and torch.equal(codes, e_codes) and torch.equal(scales, e_scales)
+                and torch.equal(out_t.view(torch.int16), e_out.view(torch.int16))):
             print(f"replay {rep} differs from the eager run", flush=True)
             return 1
     print("CAPTURE-OK", flush=True)
