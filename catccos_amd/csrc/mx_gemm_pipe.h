@@ -174,7 +174,8 @@ __global__ __launch_bounds__(256) void mx_gemm_pipe_kernel(const GemmParams p) {
     // ---- tile sequence of this workgroup ------------------------------------------------------------------
     // The two-slot kernels with the SwiGLU or the lean 16-bit store epilogue are persistent: the grid is one
     // workgroup per CU, and workgroup j of XCD x walks tiles j, j + (workgroups per XCD), ... of that XCD's
-    // contiguous run, carrying the load pipeline across tile boundaries.  The others take one tile per
+    // contiguous run (or, in fixed strides over at least a round of tiles, the XCDs take turns at blocks of
+    // consecutive tiles: interleave_xcd_walk), carrying the load pipeline across tile boundaries.  The others take one tile per
     // workgroup (the general store epilogue with its three output types and edge cases needs too many
     // registers to sit inside the loop).
     constexpr bool kPersistent = pipe_is_persistent(NSLOT, EPI);
@@ -182,9 +183,10 @@ __global__ __launch_bounds__(256) void mx_gemm_pipe_kernel(const GemmParams p) {
     const uint32_t total_tiles = m_tiles_all * p.w_tiles;
     uint32_t run_count;
     const uint32_t run_first = xcd_run(total_tiles, blockIdx.x % kXcds, run_count);
-    const uint32_t run_end = run_first + run_count;
-    const uint32_t tile_stride = kPersistent ? gridDim.x / kXcds : total_tiles;      // one tile only when not persistent
+    uint32_t run_end = run_first + run_count;
+    uint32_t tile_stride = kPersistent ? gridDim.x / kXcds : total_tiles;      // one tile only when not persistent
     uint32_t tile_id = run_first + blockIdx.x / kXcds;
+    if (kPersistent && p.tile_ctr == nullptr) interleave_xcd_walk(total_tiles, tile_id, tile_stride, run_end);
     if (tile_id >= run_end) return;
 
     // addressing of the tile whose slabs are being requested (switches two slabs before a tile boundary)

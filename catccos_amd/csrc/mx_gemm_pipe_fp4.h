@@ -105,9 +105,10 @@ __global__ __launch_bounds__(256) void mx_gemm_pipe_fp4_kernel(const GemmParams 
     const uint32_t total_tiles = m_tiles_all * p.w_tiles;
     uint32_t run_count;
     const uint32_t run_first = xcd_run(total_tiles, blockIdx.x % kXcds, run_count);
-    const uint32_t run_end = run_first + run_count;
-    const uint32_t tile_stride = kPersistent ? gridDim.x / kXcds : total_tiles;
+    uint32_t run_end = run_first + run_count;
+    uint32_t tile_stride = kPersistent ? gridDim.x / kXcds : total_tiles;      // one tile only when not persistent
     uint32_t tile_id = run_first + blockIdx.x / kXcds;
+    if (kPersistent && p.tile_ctr == nullptr) interleave_xcd_walk(total_tiles, tile_id, tile_stride, run_end);
     if (tile_id >= run_end) return;
 
     // addressing of the tile whose slabs are being requested (switches two slabs before a tile boundary)
