@@ -445,6 +445,71 @@ __device__ __forceinline__ void epilogue(const GemmParams& p, const Tile& tc, v1
     }
 }
 
+// The lean 16-bit store in whole cache lines, for the persistent two-slot kernels.  Straight from the accumulator layout
+// (epilogue above) a store instruction writes 32 bytes to each of 32 rows and a 128-byte line is complete only after four
+// such instructions.  Here the 32 rows x 128 bytes that two neighbouring weight fragments hold for one activation fragment go
+// through a 4 KiB staging area in the LDS (16-byte pieces, XOR-swizzled by row: neither the writes nor the reads conflict)
+// and come back with eight lanes on a row, so that a store instruction writes eight whole lines, non-temporal (the kernel
+// does not read its output again).  `stage` is the wavefront's own 4 KiB; a wavefront reads only what it wrote itself.
+template <int TW, int TM, int WW, int WM, int EPI, int FW, int FM>
+__device__ __forceinline__ void lean_store_lines(const GemmParams& p, const Tile& tc, v16f (&acc)[FW][FM], uint32_t ww, uint32_t wm,
+                                                 uint32_t lane, uint32_t stage) {
+    static_assert(epi_is_lean_store(EPI) && FW % 2 == 0, "16-bit store epilogues, weight fragments in pairs");
+    const uint32_t l32 = lane & 31u, lh = lane >> 5;
+    auto pack = [](float a, float b) -> uint32_t {
+        if constexpr (EPI == kEpiStoreFp16) {
+            typedef _Float16 v2h __attribute__((ext_vector_type(2)));
+            return __builtin_bit_cast(uint32_t, (v2h){(_Float16)a, (_Float16)b});
+        } else {
+            return cvt_pk_bf16(a, b);
+        }
+    };
+    // write side: row l32 of the fragment, piece (f2, qp, lh) = columns 32 f2 + 16 qp + 8 lh .. + 8 of the pair's 64
+    const uint32_t wr_row = stage + l32 * 128;
+    // read side: instruction j covers rows 8 j .. 8 j + 7, lane i row 8 j + i / 8, piece i % 8
+    const uint32_t rd_r = lane >> 3, rd_p = lane & 7u;
+    uint16_t* const c = reinterpret_cast<uint16_t*>(p.c);
+#pragma unroll
+    for (int fm = 0; fm < FM; ++fm) {
+#pragma unroll
+        for (int pr = 0; pr < FW / 2; ++pr) {
+#pragma unroll
+            for (int f2 = 0; f2 < 2; ++f2) {
+                const int fw = 2 * pr + f2;
+#pragma unroll
+                for (int qp = 0; qp < 2; ++qp) {
+                    const int q = 2 * qp;
+                    const uint32_t a0 = pack(acc[fw][fm][4 * q], acc[fw][fm][4 * q + 1]);
+                    const uint32_t a1 = pack(acc[fw][fm][4 * q + 2], acc[fw][fm][4 * q + 3]);
+                    const uint32_t b0 = pack(acc[fw][fm][4 * q + 4], acc[fw][fm][4 * q + 5]);
+                    const uint32_t b1 = pack(acc[fw][fm][4 * q + 6], acc[fw][fm][4 * q + 7]);
+                    // upper half of a <-> lower half of b: either lane ends up with eight consecutive columns of its row
+                    const auto s0 = __builtin_amdgcn_permlane32_swap(a0, b0, false, false);
+                    const auto s1 = __builtin_amdgcn_permlane32_swap(a1, b1, false, false);
+                    const uint32_t piece = 4 * f2 + 2 * qp + lh;
+                    const uint32_t addr = wr_row + ((piece ^ (l32 & 7u)) << 4);
+                    asm volatile("ds_write_b128 %0, %1" ::"v"(addr), "v"((v4i){(int)s0[0], (int)s1[0], (int)s0[1], (int)s1[1]}) : "memory");
+                }
+            }
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+            v4i v[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const uint32_t r = 8 * j + rd_r;
+                asm volatile("ds_read_b128 %0, %1" : "=v"(v[j]) : "v"(stage + r * 128 + ((rd_p ^ (r & 7u)) << 4)) : "memory");
+            }
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");       // also: the area is free for the next pair's pieces
+            const uint32_t col = tc.wt * TW + ww * (TW / WW) + pr * 64 + rd_p * 8;      // first of the lane's eight output columns
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const uint32_t mloc = wm * (TM / WM) + fm * 32 + 8 * j + rd_r;
+                if (mloc < tc.rows_valid && col < p.n)                   // n is a multiple of 8: a piece is in or out as a whole
+                    __builtin_nontemporal_store(v[j], reinterpret_cast<v4i*>(c + (size_t)(tc.row0 + mloc) * p.ldc + col));
+            }
+        }
+    }
+}
+
 // TW/TM: tile rows (weights / activations); WW x WM wavefront grid over the tile (4 or 8 wavefronts).
 // FAST: K is a whole number of slabs and scale rows are dword aligned, so the main loop carries no
 // bounds checks at all.
@@ -1060,7 +1125,9 @@ int launch_gemm_dl(const GemmParams& p, uint32_t max_m_tiles, hipStream_t s) {
 template <int FMT, int EPI, int TM, int WW, int WM, int NSLOT>
 int launch_gemm_pipe(const GemmParams& p, uint32_t max_m_tiles, hipStream_t s) {
     // tile ring, scale ring (two-slot kernels: two blocks of 16 bytes per row), next-tile mailbox, 256-byte sink of the L2 prefetch loads
-    constexpr size_t smem = NSLOT * (256 + TM) * kSlabBytes + (NSLOT == 2 ? 2 * (256 + TM) * 16 : NSLOT * (256 + TM) * 4) + 512;
+    // (+ the 16 KiB staging area of the whole-line stores, which overlays the last 512 bytes)
+    constexpr size_t smem = NSLOT * (256 + TM) * kSlabBytes + (NSLOT == 2 ? 2 * (256 + TM) * 16 : NSLOT * (256 + TM) * 4) +
+                            (pipe_stages_stores(NSLOT, EPI, WW, WM) ? 16384 : 512);
     constexpr auto kfn = mx_gemm_pipe_kernel<FMT, EPI, TM, WW, WM, NSLOT>;
     if (int rc = allow_dynamic_lds<kfn, smem>(); rc != CMX_OK) return rc;
     const uint64_t tiles = (uint64_t)max_m_tiles * p.w_tiles;
@@ -1097,7 +1164,9 @@ int launch_gemm_wreg(const GemmParams& p, uint32_t max_m_tiles, hipStream_t s) {
 
 template <int EPI, int WW, int WM>
 int launch_gemm_pipe_fp4(const GemmParams& p, uint32_t max_m_tiles, hipStream_t s) {
-    constexpr size_t smem = 2 * 512 * kSlabBytes + 2 * 512 * 16 + 512;    // tile ring, ring of two scale blocks, next-tile mailbox, sink of the L2 prefetch loads
+    // tile ring, ring of two scale blocks, next-tile mailbox and sink of the L2 prefetch loads (or the 16 KiB staging area of the
+    // whole-line stores, which overlays those 512 bytes)
+    constexpr size_t smem = 2 * 512 * kSlabBytes + 2 * 512 * 16 + (pipe_stages_stores(2, EPI, WW, WM) ? 16384 : 512);
     constexpr auto kfn = mx_gemm_pipe_fp4_kernel<EPI, WW, WM>;
     if (int rc = allow_dynamic_lds<kfn, smem>(); rc != CMX_OK) return rc;
     const uint64_t tiles = (uint64_t)max_m_tiles * p.w_tiles;

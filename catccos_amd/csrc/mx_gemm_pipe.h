@@ -119,6 +119,11 @@ __device__ __forceinline__ v8i join8(const v4i& lo, const v4i& hi) {
 //           so short that every tile streams its weights from HBM once and the load latency, not the MFMA
 //           rate, sets the pace.
 __host__ __device__ constexpr bool pipe_is_persistent(int nslot, int epi) { return nslot == 2 && epi != kEpiStore; }
+// The persistent 2 x 2 kernels with the lean 16-bit store epilogue write their output in whole lines through an LDS
+// staging area of 4 KiB per wavefront: the 16 KiB that the rings leave free, including the mailbox and the prefetch sink.
+__host__ __device__ constexpr bool pipe_stages_stores(int nslot, int epi, int ww, int wm) {
+    return pipe_is_persistent(nslot, epi) && epi_is_lean_store(epi) && ww == 2 && wm == 2;
+}
 
 // L2 prefetch distance in slabs for the persistent 2 x 2 kernels (0: none).  The workgroups that run side by side on
 // an XCD share operand panels, and without help the one that is furthest ahead pays the HBM latency of every shared
@@ -649,7 +654,15 @@ __global__ __launch_bounds__(256) void mx_gemm_pipe_kernel(const GemmParams p) {
             sm += 2;
             if (sm == nslab) {
                 fence_accumulators();           // the last MFMAs have written their accumulators
-                epilogue<TW, TM, WW, WM, EPI, FW, FM>(p, tc, acc, ww, wm, lane);
+                if constexpr (pipe_stages_stores(NSLOT, EPI, WW, WM)) {
+                    // The staging area overlays the sink of the prefetch loads: every wavefront's loads must have landed
+                    // before anyone stages.  (They are the next tile's first two slabs and their prefetches, issued a slab
+                    // ago.)  No prefetch is issued again before two barriers of the next slab, when everyone is done here.
+                    asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");
+                    lean_store_lines<TW, TM, WW, WM, EPI, FW, FM>(p, tc, acc, ww, wm, lane, lds0 + kScaleBase + kScaleRingBytes + wave * 4096);
+                } else {
+                    epilogue<TW, TM, WW, WM, EPI, FW, FM>(p, tc, acc, ww, wm, lane);
+                }
                 if (!next_ok) break;
                 tile_id = next_id;
                 tc = tq;

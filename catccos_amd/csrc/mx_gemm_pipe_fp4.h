@@ -453,7 +453,13 @@ __global__ __launch_bounds__(256) void mx_gemm_pipe_fp4_kernel(const GemmParams 
             sm += 2;
             if (sm == nslab) {
                 fence_accumulators();           // the last MFMAs have written their accumulators
-                epilogue<TW, TM, WW, WM, EPI, FW, FM>(p, tc, acc, ww, wm, lane);
+                if constexpr (pipe_stages_stores(2, EPI, WW, WM)) {
+                    // whole-line stores through the staging area that overlays the prefetch sink (see mx_gemm_pipe_kernel)
+                    asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");
+                    lean_store_lines<TW, TM, WW, WM, EPI, FW, FM>(p, tc, acc, ww, wm, lane, lds0 + kScaleBase + 2 * kScaleSlotBytes + wave * 4096);
+                } else {
+                    epilogue<TW, TM, WW, WM, EPI, FW, FM>(p, tc, acc, ww, wm, lane);
+                }
                 if (!next_ok) break;
                 tile_id = next_id;
                 tc = tq;
