@@ -192,6 +192,10 @@ __global__ __launch_bounds__(256) void mx_gemm_pipe_kernel(const GemmParams p) {
     uint32_t tile_stride = kPersistent ? gridDim.x / kXcds : total_tiles;      // one tile only when not persistent
     uint32_t tile_id = run_first + blockIdx.x / kXcds;
     if (kPersistent && p.tile_ctr == nullptr) interleave_xcd_walk(total_tiles, tile_id, tile_stride, run_end);
+    if (!kPersistent && blockIdx.x < total_tiles) {
+        tile_id = tile_of_workgroup(total_tiles);
+        run_end = total_tiles;
+    }
     if (tile_id >= run_end) return;
 
     // addressing of the tile whose slabs are being requested (switches two slabs before a tile boundary)
