@@ -67,3 +67,31 @@ def test_grouped_sweep(counts, n, k):
         deq, deq_g = O.mx_dequant(host(codes), host(scales)), O.mx_dequant(gq, gs)
         bound = 0.13 * np.abs(deq_g) + 2.0 ** -5 * np.abs(deq_g).max(axis=1, keepdims=True) + 1e-6
         assert np.all(np.abs(deq - deq_g) <= bound)
+
+
+@pytest.mark.parametrize("fmt", ["E4M3", "E2M1"])
+@pytest.mark.parametrize("out", ["bf16", "fp16"])
+def test_output_pitch_and_edges_are_left_alone(fmt, out):
+    """The persistent kernels store their 16-bit output in whole lines through the LDS.  With an output pitch wider than
+    n, a ragged last row tile and a ragged last column tile, every element inside equals the tight-pitch call bit for bit
+    and every element outside keeps its poison."""
+    from catccos_amd import _lib, ops
+    m, n, k, ldc, pad_rows = 300, 520, 1024, 536, 3
+    rng = np.random.default_rng(77)
+    if fmt == "E2M1":
+        aq, asc = O.mx_quant(rng.uniform(-2, 2, (m, k)).astype(np.float32), "E2M1")
+        bq, bsc = O.mx_quant(rng.uniform(-2, 2, (n, k)).astype(np.float32), "E2M1")
+        aq, bq = O.pack_fp4(aq), O.pack_fp4(bq)
+    else:
+        aq, asc = O.mx_quant(O.bf16_round(rng.standard_normal((m, k)).astype(np.float32)), "E4M3")
+        bq, bsc = O.mx_quant(O.bf16_round(rng.standard_normal((n, k)).astype(np.float32)), "E4M3")
+    a, a_s, b, b_s = dev(aq), dev(asc), dev(bq), dev(bsc)
+    tight = ops.mx_gemm(a, a_s, b, b_s, k, fmt, out)
+    wide = torch.full((m + pad_rows, ldc), 0x7FC1, dtype=torch.int16, device="cuda")
+    lib = _lib.load()
+    _lib.check(lib.cmx_mx_gemm(a.data_ptr(), a.stride(0), a_s.data_ptr(), a_s.stride(0), b.data_ptr(), b.stride(0), b_s.data_ptr(),
+                               b_s.stride(0), wide.data_ptr(), ldc, m, n, k, ops.FMT[fmt], ops.OUT[out],
+                               torch.cuda.current_stream().cuda_stream))
+    torch.cuda.synchronize()
+    assert torch.equal(wide[:m, :n], tight.view(torch.int16))
+    assert bool((wide[:m, n:] == 0x7FC1).all()) and bool((wide[m:] == 0x7FC1).all())
