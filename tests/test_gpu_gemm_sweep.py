@@ -95,3 +95,31 @@ def test_output_pitch_and_edges_are_left_alone(fmt, out):
     torch.cuda.synchronize()
     assert torch.equal(wide[:m, :n], tight.view(torch.int16))
     assert bool((wide[:m, n:] == 0x7FC1).all()) and bool((wide[m:] == 0x7FC1).all())
+
+
+@pytest.mark.parametrize("fmt", ["E4M3", "E2M1"])
+def test_grouped_output_pitch_and_edges_are_left_alone(fmt):
+    """The same for the grouped matmul (ragged groups, one empty, rows past the groups): inside bit-equal to the
+    tight-pitch call, outside untouched."""
+    from catccos_amd import ops
+    counts, n, k, ldc, spare = [700, 0, 900, 650], 520, 1024, 536, 5
+    m = sum(counts)
+    rng = np.random.default_rng(78)
+    if fmt == "E2M1":
+        aq, asc = O.mx_quant(rng.uniform(-2, 2, (m + spare, k)).astype(np.float32), "E2M1")
+        ws_ = [O.mx_quant(rng.uniform(-2, 2, (n, k)).astype(np.float32), "E2M1") for _ in counts]
+        aq = O.pack_fp4(aq)
+        wq = np.stack([O.pack_fp4(q) for q, _ in ws_])
+    else:
+        aq, asc = O.mx_quant(O.bf16_round(rng.standard_normal((m + spare, k)).astype(np.float32)), "E4M3")
+        ws_ = [O.mx_quant(O.bf16_round(rng.standard_normal((n, k)).astype(np.float32)), "E4M3", "lut") for _ in counts]
+        wq = np.stack([q for q, _ in ws_])
+    wsc = np.stack([s for _, s in ws_])
+    a, a_s, w, w_s = dev(aq), dev(asc), dev(wq), dev(wsc)
+    cnt = torch.tensor(counts, dtype=torch.int32, device="cuda")
+    tight = ops.mx_gmm(a, a_s, w, w_s, cnt, k, fmt)
+    wide = torch.full((m + spare, ldc), 0x7FC1, dtype=torch.int16, device="cuda")
+    ops.mx_gmm(a, a_s, w, w_s, cnt, k, fmt, c=wide.view(torch.bfloat16)[:, :n])
+    torch.cuda.synchronize()
+    assert torch.equal(wide[:m, :n], tight.view(torch.int16)[:m])
+    assert bool((wide[:, n:] == 0x7FC1).all()) and bool((wide[m:] == 0x7FC1).all())
