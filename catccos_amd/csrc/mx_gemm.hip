@@ -993,13 +993,23 @@ __global__ __launch_bounds__(256) void gmm_prepare_kernel(const int32_t* __restr
         const int32_t c = sizes[i];
         return c > 0 ? (unsigned long long)c : 0ull;
     };
+    // inclusive scan of part[0..255] in place: within each wavefront by lane shuffles, then the three wavefront totals
+    // before it added to every element (two barriers instead of sixteen)
     auto scan256 = [&](auto* part) {
-        for (uint32_t d = 1; d < 256; d <<= 1) {
-            const auto v = threadIdx.x >= d ? part[threadIdx.x - d] : 0;
-            __syncthreads();
-            part[threadIdx.x] += v;
-            __syncthreads();
+        auto v = part[threadIdx.x];
+        const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
+#pragma unroll
+        for (int d = 1; d < 64; d <<= 1) {
+            const auto u = __shfl_up(v, d);
+            if (lane >= (uint32_t)d) v += u;
         }
+        part[threadIdx.x] = v;
+        __syncthreads();
+        decltype(v) before = 0;
+        for (uint32_t w = 0; w < wave; ++w) before += part[64 * w + 63];
+        __syncthreads();
+        part[threadIdx.x] = v + before;
+        __syncthreads();
     };
     unsigned long long r = 0;
     for (uint32_t i = lo; i < hi; ++i) r += size_of(i);
